@@ -707,7 +707,7 @@ pipe_done:
             // One chunk.  The compiler's wait-count pass works on merged states: every edge INTO a block contributes what may still be in flight there.  A trip of 2 NB tiles
             // that can be left in the middle (`if (T >= ntile) goto done`, which the structuriser routes through the loop header) handed the header the ring as the allocator
             // had it named at that exit — other registers than at the bottom of the trip — and the first blocks of every trip then waited for "pending" loads into registers
-            // they use as temporaries: vmcnt(1), (4), (7), (10) ... in front of their LDS reads, a drain of the 8-block ring per trip (ISA of round 5; tools_dev/scan_vmcnt.py
+            // they use as temporaries: vmcnt(1), (4), (7), (10) ... in front of their LDS reads, a drain of the 8-block ring per trip (ISA of round 5
             // lists such waits).  So: whole trips in a loop that has ONE exit, the bottom, and the row's last ntile % (2 NB) tiles as straight-line code behind it.
             const int nfull = ntile / (2 * NB) * (2 * NB);
             for (int T0 = 0; T0 < nfull; T0 += 2 * NB) {

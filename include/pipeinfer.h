@@ -38,6 +38,12 @@ LLAMA_API int  pipeinfer_context_set_segments(struct llama_context * ctx, int la
  * the PipeInfer driver keeps a non-speculative and one or more speculative runs queued behind the run in flight (speculative.cpp:1182-1275). */
 LLAMA_API int  pipeinfer_context_set_coalescing(struct llama_context * ctx, int max_tokens);
 /* 0: launch the decode kernels one by one instead of replaying the captured HIP graph (profiling / per-kernel event timing) */
+/* Hybrid models (a folder with config.json + model.safetensors, bfloat16 weights).  precision: 0 = serving precision (activations rounded to bfloat16 where they enter a matrix
+ * product, fp32 accumulation; norms, scores, states, router in fp32), 1 = every product in fp32.  state slots: how many sequences a context whose model has recurrent layers keeps
+ * alive at once (default 8); llama_kv_cache_seq_rm(seq, -1, -1) gives a sequence's slot back.  Both before the first decode. */
+LLAMA_API int pipeinfer_context_set_precision(struct llama_context * ctx, int exact);
+LLAMA_API int pipeinfer_context_set_state_slots(struct llama_context * ctx, int n_slots);
+LLAMA_API int pipeinfer_get_state_slots_used(struct llama_context * ctx);
 LLAMA_API void pipeinfer_context_set_graphs(struct llama_context * ctx, int enable);
 LLAMA_API const char * pipeinfer_context_error(struct llama_context * ctx);
 LLAMA_API int32_t pipeinfer_model_n_layer(const struct llama_model * model);

@@ -29,7 +29,7 @@ extern "C" {
 #define PI_API __attribute__((visibility("default")))
 
 /* ggml tensor type ids (ggml.h enum ggml_type) */
-enum pi_type { PI_F32 = 0, PI_F16 = 1, PI_Q4_0 = 2, PI_Q4_1 = 3, PI_Q5_0 = 6, PI_Q5_1 = 7, PI_Q8_0 = 8, PI_Q8_1 = 9, PI_Q2_K = 10, PI_Q3_K = 11, PI_Q4_K = 12, PI_Q5_K = 13, PI_Q6_K = 14, PI_Q8_K = 15 };
+enum pi_type { PI_F32 = 0, PI_F16 = 1, PI_Q4_0 = 2, PI_Q4_1 = 3, PI_Q5_0 = 6, PI_Q5_1 = 7, PI_Q8_0 = 8, PI_Q8_1 = 9, PI_Q2_K = 10, PI_Q3_K = 11, PI_Q4_K = 12, PI_Q5_K = 13, PI_Q6_K = 14, PI_Q8_K = 15, PI_BF16 = 30 /* bfloat16 rows as a safetensors checkpoint holds them (dense operators below) */ };
 
 typedef struct pi_weight pi_weight;    /* a weight matrix resident in HBM in the kernel-friendly layout */
 
@@ -173,6 +173,36 @@ PI_API int pi_op_clamp(float * x_dev, float lo, float hi, int64_t n, void * stre
 /* per token: ids/logits of the k largest (logit desc, id asc), max logit and sum_i expf(l_i - max) over the full vocab */
 PI_API size_t pi_op_topk_scratch_bytes(int n_tok);                  /* caller-owned scratch, one per stream */
 PI_API int pi_op_topk(const float * logits_dev, int n_vocab, int n_tok, int k, int32_t * ids_dev, float * vals_dev, float * sumexp_dev, void * scratch_dev, void * stream);
+
+/* ---- dense bfloat16 matrices and the operators of hybrid blocks (recurrent / low-rank-attention mixers, routed feed-forwards) --------------------------------------
+ * Weights are PI_BF16 pi_weights ([rows][K] as stored, pi_weight_upload(PI_BF16, K, rows, ...)); activations, norms, scores, states and outputs are fp32.
+ * exact = 0: activations are rounded to bfloat16 where they enter a matrix product (fp32 accumulation); exact = 1: nothing is rounded, every product is an fp32 fma. */
+enum pi_act { PI_ACT_NONE = 0, PI_ACT_SILU = 1, PI_ACT_SIGMOID = 2, PI_ACT_RELU_SQR = 3 };
+/* out[t][:] = widen(table[tokens[t]]) * scale */
+PI_API int pi_op_embed(const pi_weight * table, const int32_t * tokens_dev, int n_tok, float scale, float * out_dev, void * stream);
+/* out[t][r] = act(W[r] . x[t]); rows [0, rows_a) take act_a, the others act_b (projections that share their input are one matrix and one launch); strides in floats */
+PI_API int pi_op_dense(const pi_weight * w, const float * x_dev, int64_t x_stride, int n_tok, float * out_dev, int64_t out_stride, int act_a, int64_t rows_a, int act_b, int exact, void * stream);
+/* y = x / sqrt(mean(x^2) + eps) * (w + w_offset) [* gate]; out = [residual +] mult * y.  to_cells != 0: row t is written to row cell(t) of `out` (dyn_dev as for pi_op_attention_ex) */
+PI_API int pi_op_rms_scale(const float * x_dev, int64_t x_stride, const float * w_dev, float w_offset, float eps, int n, int n_tok, const float * gate_dev, int64_t gate_stride,
+                           const float * residual_dev, int64_t residual_stride, float mult, float * out_dev, int64_t out_stride, const int32_t * dyn_dev, int to_cells, void * stream);
+/* Linear attention with a per-head decay: S <- decay[h] * S + k v^T, o = S^T q, token by token.  q / k: [n_tok][heads * dim], v: [n_tok][heads * vdim], all `stride` floats apart;
+ * state_dev: [slots][heads][dim][vdim] fp32; rec_dev[t]: the slot of token t's sequence, | 1 << 30 on a token whose sequence starts from a zero state; tokens of one slot are
+ * consecutive and at most max_segments slots occur in a pass */
+PI_API int pi_op_linear_attention(const float * q_dev, const float * k_dev, const float * v_dev, int64_t stride, int heads, int dim, int vdim, const float * decay_dev, float * state_dev,
+                                  const int32_t * rec_dev, int n_tok, int max_segments, float * out_dev, int64_t out_stride, void * stream);
+PI_API int pi_op_copy_f32(const float * src_dev, float * dst_dev, int64_t n, void * stream);
+/* Attention over a cache of latents c [cells][rank] fp32 shared by all heads: k = W_uk c, v = W_uv c per head, never materialised (W_uk is folded into the query, W_uv applied to
+ * the weighted sum of latents); score = q . k * scale; soft-max whose denominator also holds exp(sink[h]).  mask_dev / n_kv / dyn_dev as for pi_op_attention_ex (single run). */
+PI_API int pi_op_latent_attention(const float * q_dev, int64_t q_stride, const float * cache_dev, const uint32_t * mask_dev, const pi_weight * w_uk, const pi_weight * w_uv, const float * sink_dev,
+                                  float scale, int heads, int dim, int vdim, int rank, int n_tok, int n_kv, float * out_dev, int64_t out_stride, const int32_t * dyn_dev, void * stream);
+PI_API int pi_op_latent_attention_reserve(void);                   /* once per process, outside graph capture: LDS limit for long contexts */
+PI_API int pi_op_latent_attention_max_cells(int rank);             /* longest context the kernel serves at this latent width */
+/* Router of a mixture of experts: scores = softmax(W_router x) over all outputs; the `top` outputs with the largest score + correction are chosen (lowest index wins a tie); their
+ * weights are the scores themselves.  sel_dev / selw_dev: [n_tok][top] */
+PI_API int pi_op_moe_route(const pi_weight * router, const float * correction_dev, const float * x_dev, int64_t x_stride, int n_tok, int top, int exact, int32_t * sel_dev, float * selw_dev, void * stream);
+/* out[t] = sum over the chosen outputs e of weight * (e < n_exp ? W_down[e] relu(W_up[e] x[t])^2 : x[t]); w_up: [n_exp * ff][width], w_down: [n_exp * width][ff]; up_dev: scratch [n_tok][top][ff] */
+PI_API int pi_op_moe_experts(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, const float * x_dev, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
+                             int exact, float * up_dev, float * out_dev, int64_t out_stride, void * stream);
 
 #ifdef __cplusplus
 }

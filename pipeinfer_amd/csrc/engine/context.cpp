@@ -40,7 +40,7 @@ llama_context::~llama_context() {
     if (hop_host) (void) hipHostFree(hop_host);
     pi_free(hop_dev);
     pi_free(abort_dev);
-    void * bufs[] = { k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
+    void * bufs[] = { lat_cache, rec_state, rec_dev, h_in, h_att, h_out, moe_w, moe_up, moe_sel, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
     for (void * b : bufs) pi_free(b);
     if (rope) pi_rope_table_free(rope);
     if (stream) (void) hipStreamDestroy(stream);
@@ -49,6 +49,7 @@ llama_context::~llama_context() {
 namespace pi {
 
 static size_t kv_bytes_per_cell(const llama_context * ctx) {
+    if (ctx->model->hparams.hybrid_arch()) { size_t b = 0; for (const auto & l : ctx->model->hparams.hybrid) if (l.cache_index >= 0) b += (size_t) 4 * l.kv_rank; return b; }
     return (size_t) 2 * 2 * ctx->model->hparams.n_embd_gqa() * (size_t) (ctx->l1 - ctx->l0);
 }
 
@@ -86,10 +87,63 @@ bool context_prepare(llama_context * ctx, std::string & err) {
     if (ctx->seg_layers > 0 && !context_precapture(ctx, std::max(8, ctx->coalesce_max.load()))) { ctx->last_error = "graph capture of the narrow pass widths failed: " + ctx->last_error; err = ctx->last_error; return false; }
     return true;
 }
+// device state of a hybrid model: latent caches and recurrent states at per-layer offsets, fp32 scratch rows for the widest layer
+static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
+    llama_model * m = ctx->model;
+    const pi_hparams & hp = m->hparams;
+    if (ctx->seg_layers > 0 || ctx->remote || !ctx->is_first || !ctx->is_last || ctx->l0 != 0 || ctx->l1 != hp.n_layer) {
+        err = "a hybrid model runs as one stage on one GPU: segmented launches, run coalescing and layer-split pipelines are for the GGUF architectures (its recurrent layers keep ONE state per sequence, which a cancelled or re-ordered run cannot give back)";
+        return false;
+    }
+    const int64_t t0 = time_us();
+    if (!m->ensure_loaded_hybrid(err)) return false;
+    ctx->t_load_us += time_us() - t0;
+    if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) { err = "hipStreamCreate failed"; return false; }
+    auto dev = [&](size_t bytes) -> void * { void * p = pi_malloc(std::max<size_t>(bytes, 16)); if (!p) err = pi_last_error(); return p; };
+    const int nb = ctx->n_batch, width = hp.n_embd;
+    size_t lat = 0, rec = 0, in_w = 1, att_w = 1, up_w = 1, sel_w = 1;
+    ctx->lat_off.assign(hp.hybrid.size(), 0); ctx->rec_off.assign(hp.hybrid.size(), 0);
+    if (hp.n_recurrent() > 0) ctx->slots.reset(new state_slots(std::max(1, ctx->n_state_slots)));
+    for (size_t i = 0; i < hp.hybrid.size(); i++) {
+        const pi_hybrid_layer & H = hp.hybrid[i];
+        if (H.cache_index >= 0) {
+            if (ctx->n_ctx > pi_op_latent_attention_max_cells(H.kv_rank)) { err = "n_ctx = " + std::to_string(ctx->n_ctx) + " is beyond the latent-attention kernel at kv_rank " + std::to_string(H.kv_rank) + " (one score row per workgroup in LDS: n_ctx <= " + std::to_string(pi_op_latent_attention_max_cells(H.kv_rank)) + ")"; return false; }
+            ctx->lat_off[i] = lat; lat += (size_t) ctx->n_ctx * H.kv_rank;
+        }
+        if (H.state_index >= 0) { ctx->rec_off[i] = rec; rec += (size_t) ctx->slots->size() * H.heads * H.dim * H.vdim; }
+        in_w = std::max(in_w, (size_t) H.in_rows()); att_w = std::max(att_w, (size_t) H.heads * H.vdim);
+        if (H.has_mlp) { up_w = std::max(up_w, (size_t) H.top * std::max(H.ff, 1)); sel_w = std::max(sel_w, (size_t) H.top); }
+    }
+    if (!(ctx->lat_cache = (float *) dev(lat * 4)) || !(ctx->rec_state = (float *) dev(rec * 4))) return false;
+    pi_memset(ctx->lat_cache, 0, std::max<size_t>(lat * 4, 16), nullptr); pi_memset(ctx->rec_state, 0, std::max<size_t>(rec * 4, 16), nullptr);
+    if (!(ctx->x = (float *) dev((size_t) 4 * nb * width)) || !(ctx->nx = (float *) dev((size_t) 4 * nb * width)) || !(ctx->h_out = (float *) dev((size_t) 4 * nb * width)) ||
+        !(ctx->h_in = (float *) dev((size_t) 4 * nb * in_w)) || !(ctx->h_att = (float *) dev((size_t) 4 * nb * att_w)) || !(ctx->moe_up = (float *) dev((size_t) 4 * nb * up_w)) ||
+        !(ctx->moe_w = (float *) dev((size_t) 4 * nb * sel_w)) || !(ctx->moe_sel = (int32_t *) dev((size_t) 4 * nb * sel_w)) || (ctx->slots && !(ctx->rec_dev = (int32_t *) dev((size_t) 4 * nb))) ||
+        !(ctx->tokens_dev = (int32_t *) dev((size_t) 4 * nb)) || !(ctx->pos_dev = (int32_t *) dev((size_t) 4 * nb)) || !(ctx->dyn_dev = (int32_t *) dev((size_t) 4 * (4 + 2 * nb))))
+        return false;
+    {   // abort word + cancel flags + the control stream cancels travel on
+        if (!(ctx->abort_dev = (int32_t *) dev(256))) return false;
+        pi_memset(ctx->abort_dev, 0, 256, nullptr);
+        if (hipHostMalloc((void **) &ctx->abort_host, 256 * sizeof(int32_t), hipHostMallocDefault) != hipSuccess) { err = "hipHostMalloc(abort flags) failed"; return false; }
+        memset(ctx->abort_host, 0, 256 * sizeof(int32_t));
+        if (hipStreamCreateWithFlags(&ctx->ctl_stream, hipStreamNonBlocking) != hipSuccess) { err = "hipStreamCreate(control) failed"; return false; }
+    }
+    ctx->use_graphs = ctx->use_graphs && getenv("PI_NO_GRAPHS") == nullptr;
+    if (pi_op_latent_attention_reserve() != 0) { err = pi_last_error(); return false; }
+    ctx->mask_cap_words = (size_t) nb * ((ctx->n_ctx + 31) / 32);
+    if (!(ctx->mask_dev = (uint32_t *) dev(ctx->mask_cap_words * 4))) return false;
+    if (!(ctx->logits_dev = (float *) dev((size_t) 4 * nb * hp.n_vocab)) || !(ctx->topk_ids_dev = (int32_t *) dev((size_t) 4 * nb * 8)) ||
+        !(ctx->topk_vals_dev = (float *) dev((size_t) 4 * nb * 8)) || !(ctx->topk_sum_dev = (float *) dev((size_t) 4 * nb)) || !(ctx->topk_scratch_dev = dev(pi_op_topk_scratch_bytes(nb))))
+        return false;
+    if (hipDeviceSynchronize() != hipSuccess) { err = "hipDeviceSynchronize failed after allocation"; return false; }
+    return true;
+}
+
 static bool context_prepare_impl(llama_context * ctx, std::string & err) {
     llama_model * m = ctx->model;
     const pi_hparams & hp = m->hparams;
     if (pi_device_init(m->device) != 0) { err = pi_last_error(); return false; }
+    if (hp.hybrid_arch()) return context_prepare_hybrid(ctx, err);
     const int64_t t0 = time_us();
     // a context whose n_batch-bounded widest pass stays below the matrix-core kernel's first width never reads the tile-major copies: do not make them
     if (!m->ensure_loaded(ctx->l0, ctx->l1, ctx->is_first, ctx->is_last, ctx->n_batch >= pi_op_mmq_min_tokens(), err)) return false;
@@ -218,10 +272,53 @@ static bool mul_mat_grouped(int n, const pi_weight * const * ws, const void * co
     return true;
 }
 
+// A hybrid model's pass: per layer  x += m * N1(mixer(x)),  x += m * N2(moe(x))  — the norm sits on the sublayer's output, the sublayers read x itself; everything between the
+// matrix products is fp32.  Kernel sequence: fused input projection (activations in its epilogue) -> mixer kernel -> output projection -> norm + scale + residual; router ->
+// experts -> norm + scale + residual; final norm -> logits against the embedding table itself.
+static bool forward_hybrid(llama_context * ctx, int n_tok, int n_kv) {
+    llama_model * m = ctx->model;
+    const pi_hparams & hp = m->hparams;
+    hipStream_t s = ctx->stream;
+    const int width = hp.n_embd, ex = ctx->exact;
+    const float eps = hp.f_norm_rms_eps, rm = hp.residual_mult;
+    float * x = ctx->x, * P = ctx->h_in, * A = ctx->h_att, * Y = ctx->h_out;
+    OP_OK(pi_op_embed(m->tok_embd, ctx->tokens_dev, n_tok, hp.embed_scale, x, s));
+    for (size_t il = 0; il < hp.hybrid.size(); il++) {
+        const pi_hybrid_layer & H = hp.hybrid[il];
+        const pi_hybrid_weights & W = m->hweights[(size_t) H.weights];
+        const int64_t hd = (int64_t) H.heads * H.dim, hv = (int64_t) H.heads * H.vdim, pw = H.in_rows();
+        if (H.mixer == PI_MIXER_LATENT_ATTENTION) {
+            float * cache = ctx->lat_cache + ctx->lat_off[il];
+            OP_OK(pi_op_dense(W.w_in, x, width, n_tok, P, pw, PI_ACT_NONE, pw, PI_ACT_NONE, ex, s));                                               // q | W_dkv h
+            OP_OK(pi_op_rms_scale(P + hd, pw, W.mix_norm, 0.0f, eps, H.kv_rank, n_tok, nullptr, 0, nullptr, 0, 1.0f, cache, H.kv_rank, ctx->dyn_dev, 1, s));   // the latent, into its cell
+            OP_OK(pi_op_latent_attention(P, pw, cache, ctx->mask_dev, W.w_uk, W.w_uv, W.sink, H.scale, H.heads, H.dim, H.vdim, H.kv_rank, n_tok, n_kv, A, hv, ctx->dyn_dev, s));
+        } else {
+            float * state = ctx->rec_state + ctx->rec_off[il];
+            OP_OK(pi_op_dense(W.w_in, x, width, n_tok, P, pw, PI_ACT_SILU, 2 * hd + hv, PI_ACT_SIGMOID, ex, s));                                   // silu(q | k | v) | sigmoid(g)
+            OP_OK(pi_op_linear_attention(P, P + hd, P + 2 * hd, pw, H.heads, H.dim, H.vdim, W.decay, state, ctx->rec_dev, n_tok, ctx->slots->size(), A, hv, s));
+            OP_OK(pi_op_rms_scale(A, hv, W.mix_norm, 0.0f, eps, (int) hv, n_tok, P + 2 * hd + hv, pw, nullptr, 0, 1.0f, A, hv, nullptr, 0, s));    // norm over all heads, * gate
+        }
+        trace(ctx, "mix", (int) il, A, hv, n_tok);
+        OP_OK(pi_op_dense(W.w_o, A, hv, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+        OP_OK(pi_op_rms_scale(Y, width, W.norm1, 1.0f, eps, width, n_tok, nullptr, 0, x, width, rm, x, width, nullptr, 0, s));
+        if (H.has_mlp) {
+            OP_OK(pi_op_moe_route(W.router, W.correction, x, width, n_tok, H.top, ex, ctx->moe_sel, ctx->moe_w, s));
+            OP_OK(pi_op_moe_experts(W.e_up, W.e_down, H.n_expert, H.ff, x, width, ctx->moe_sel, ctx->moe_w, n_tok, H.top, ex, ctx->moe_up, Y, width, s));
+            OP_OK(pi_op_rms_scale(Y, width, W.norm2, 1.0f, eps, width, n_tok, nullptr, 0, x, width, rm, x, width, nullptr, 0, s));
+        }
+        trace(ctx, "lout", (int) il, x, width, n_tok);
+    }
+    OP_OK(pi_op_rms_scale(x, width, m->output_norm, 1.0f, eps, width, n_tok, nullptr, 0, nullptr, 0, 1.0f, ctx->nx, width, nullptr, 0, s));
+    OP_OK(pi_op_dense(m->tok_embd, ctx->nx, width, n_tok, ctx->logits_dev, hp.n_vocab, PI_ACT_NONE, hp.n_vocab, PI_ACT_NONE, ex, s));
+    OP_OK(pi_op_topk(ctx->logits_dev, hp.n_vocab, n_tok, 8, ctx->topk_ids_dev, ctx->topk_vals_dev, ctx->topk_sum_dev, ctx->topk_scratch_dev, s));
+    return true;
+}
+
 // layers [la, lb) of this stage; `head`: the embedding lookup goes first, `tail`: final norm + lm_head + top-k go last
 static bool forward(llama_context * ctx, int n_tok, int kv_head, int n_kv, int la, int lb, bool head, bool tail, bool multi = false) {
     llama_model * m = ctx->model;
     const pi_hparams & hp = m->hparams;
+    if (hp.hybrid_arch()) return forward_hybrid(ctx, n_tok, n_kv);
     const int n_embd = hp.n_embd, n_gqa = hp.n_embd_gqa(), n_ff = hp.n_ff, hd = hp.head_dim();
     hipStream_t s = ctx->stream;
     float * x = ctx->x, * x2 = ctx->x2;
@@ -386,6 +483,7 @@ static bool launch_inputs(llama_context * ctx, int n_tokens, const void * meta, 
               hipMemcpyAsync(ctx->pos_dev, h_pos, (size_t) 4 * n_tokens, hipMemcpyHostToDevice, s) == hipSuccess &&
               hipMemcpyAsync(ctx->dyn_dev, h_dyn, 16 + 4 * n_table, hipMemcpyHostToDevice, s) == hipSuccess &&
               hipMemcpyAsync(ctx->mask_dev, h_mask, (size_t) 4 * n_tokens * words, hipMemcpyHostToDevice, s) == hipSuccess;
+    if (ok && ctx->rec_dev) ok = hipMemcpyAsync(ctx->rec_dev, h_mask + (size_t) n_tokens * words, (size_t) 4 * n_tokens, hipMemcpyHostToDevice, s) == hipSuccess;     // (behind the mask rows: the state slot of every token)
     if (ok && x_in) ok = hop_store(ctx->x, x_in, (size_t) 4 * n_tokens * ctx->model->hparams.n_embd, s);      // device (this stage's ring: a kernel) or host (staged transport: a copy)
     if (!ok) ctx->last_error = "H2D of batch metadata failed";
     return ok;
@@ -717,10 +815,37 @@ pi_run * context_start(llama_context * ctx, const llama_batch & batch_in, int & 
     }
     const int n_kv = ctx->cells->n_attend();
     const int words = (ctx->n_ctx + 31) / 32;                                   // fixed row stride of the visibility bitmap
-    const size_t meta_bytes = (size_t) n_tokens * 8 + 16 + (size_t) n_tokens * words * 4;
+    // models with recurrent layers: the state slot of every token's sequence rides behind the mask rows.  A token belongs to ONE sequence there, and a sequence's tokens are
+    // consecutive in the batch (the recurrence walks them in order inside one workgroup).
+    const bool recurrent = ctx->slots != nullptr;
+    std::vector<int32_t> rec; std::vector<int> fresh_taken;
+    if (recurrent) {
+        rec.resize((size_t) n_tokens);
+        std::set<int> closed; int cur = -1, cur_slot = -1; bool bad = false, full = false;
+        for (int i = 0; i < n_tokens && !bad && !full; i++) {
+            if (n_seq_id[i] != 1) { bad = true; break; }
+            const int sq = seq_id[i][0];
+            if (sq != cur) {
+                if (cur >= 0) closed.insert(cur);
+                if (closed.count(sq)) { bad = true; break; }
+                cur = sq; cur_slot = ctx->slots->acquire(sq);
+                if (cur_slot < 0) { full = true; break; }
+                const bool fresh = ctx->slots->take_fresh(cur_slot);
+                if (fresh) fresh_taken.push_back(cur_slot);
+                rec[(size_t) i] = cur_slot | (fresh ? (1 << 30) : 0);
+            } else rec[(size_t) i] = cur_slot;
+        }
+        if (bad || full) {
+            for (int sl : fresh_taken) ctx->slots->mark_fresh(sl);
+            ctx->cells->release_cells(kv_head, n_tokens);
+            if (bad) { ctx->last_error = "a model with recurrent layers takes tokens of ONE sequence each, a sequence's tokens next to each other in the batch"; return nullptr; }
+            ctx->last_error = "no free state slot: " + std::to_string(ctx->slots->size()) + " sequences are live (pipeinfer_context_set_state_slots)"; rc = 1; return nullptr;
+        }
+    }
+    const size_t meta_bytes = (size_t) n_tokens * 8 + 16 + (size_t) n_tokens * words * 4 + (recurrent ? (size_t) n_tokens * 4 : 0);
     pi_run * run = acquire_run(ctx, n_tokens, meta_bytes);
     // (a run that cannot be started gives the cells find_slot just allotted back: nothing was or will be written to them)
-    auto give_back = [&]() { ctx->cells->release_cells(kv_head, n_tokens); };
+    auto give_back = [&]() { ctx->cells->release_cells(kv_head, n_tokens); for (int sl : fresh_taken) ctx->slots->mark_fresh(sl); };
     if (!run) { ctx->last_error = "out of pinned host memory"; give_back(); return nullptr; }
     run->batch_id = batch_in.batch_id; run->n_tokens = n_tokens; run->t_start_us = time_us(); run->sink = nullptr;
     run->run_id = (++ctx->run_counter) & 0x3fffffff; run->kv_head = kv_head; run->n_kv = n_kv;
@@ -744,6 +869,7 @@ pi_run * context_start(llama_context * ctx, const llama_batch & batch_in, int & 
     h_dyn[0] = kv_head; h_dyn[1] = n_kv; h_dyn[2] = n_tokens; h_dyn[3] = 0;
     ctx->cells->build_mask(n_kv, n_tokens, pos, n_seq_id, seq_id, h_mask, words);
     ctx->cells->post_decode(n_tokens);
+    if (recurrent) memcpy(h_mask + (size_t) n_tokens * words, rec.data(), (size_t) 4 * n_tokens);
 
     run->meta_bytes = meta_bytes;
     if (ctx->run_tap) ctx->run_tap(ctx->run_tap_user, run->run_id, run->batch_id, n_tokens, run->meta_host, meta_bytes, nullptr);

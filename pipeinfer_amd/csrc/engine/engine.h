@@ -24,11 +24,14 @@
 #include "../../../include/pipeinfer_ops.h"
 #include "gguf.h"
 #include "kv_cells.h"
+#include "safetensors.h"
+#include "state_slots.h"
 #include "vocab.h"
 #include "../kernels/kernel_timing.h"
 
 // LLAMA and FALCON have their own blocks in forward(); the others are one generic sequential block (norm -> attention -> + -> norm -> MLP -> +) described by pi_block below
-enum pi_arch { PI_ARCH_LLAMA = 0, PI_ARCH_FALCON = 1, PI_ARCH_BAICHUAN = 2, PI_ARCH_STARCODER = 3, PI_ARCH_REFACT = 4, PI_ARCH_BLOOM = 5, PI_ARCH_MPT = 6, PI_ARCH_STABLELM = 7, PI_ARCH_PERSIMMON = 8 };
+enum pi_arch { PI_ARCH_LLAMA = 0, PI_ARCH_FALCON = 1, PI_ARCH_BAICHUAN = 2, PI_ARCH_STARCODER = 3, PI_ARCH_REFACT = 4, PI_ARCH_BLOOM = 5, PI_ARCH_MPT = 6, PI_ARCH_STABLELM = 7, PI_ARCH_PERSIMMON = 8,
+               PI_ARCH_FASOVIK = 9 /* a hybrid model: a list of layers, each with its own mixer (pi_hybrid_layer), read from config.json + model.safetensors */ };
 
 // what the reference's build_* functions differ in (llama.cpp:3985-4104 baichuan, 4229-4327 starcoder, 4540-4630 refact, 4632-4725 bloom, 4727-4825 mpt, 4827-4939 stablelm)
 struct pi_block {
@@ -42,15 +45,41 @@ struct pi_block {
     float clamp_kqv = 0.0f;
 };
 
+// One layer of a hybrid model.  The mixer is one of the mechanisms below, each with its sizes and constants as the model's description gives them; the feed-forward is a
+// mixture of experts (or absent).  A layer may use another layer's tensors (`weights`) while keeping a cache / state of its own.
+enum pi_mixer_kind { PI_MIXER_LATENT_ATTENTION = 0,   // keys / values are up-projections of one cached low-rank latent, no positions, causal, soft-max with a per-head sink
+                     PI_MIXER_LIGHTNING = 1 };        // linear attention with a per-head decay: a [dim][vdim] state per head and sequence
+struct pi_hybrid_layer {
+    pi_mixer_kind mixer = PI_MIXER_LATENT_ATTENTION;
+    int weights = 0;                                  // index of the layer that owns the tensors (its own index unless shared)
+    int heads = 0, dim = 0, vdim = 0, kv_rank = 0;
+    float scale = 1.0f;                               // latent attention: factor on q . k
+    std::vector<float> decay;                         // lightning: per head
+    bool has_mlp = false; int n_expert = 0, n_identity = 0, top = 0, ff = 0;
+    int cache_index = -1, state_index = -1;           // ordinal among the layers that keep a latent cache / a recurrent state
+    int in_rows() const { return mixer == PI_MIXER_LIGHTNING ? 2 * heads * dim + 2 * heads * vdim : heads * dim + kv_rank; }     // rows of the fused input projection
+};
+struct pi_hybrid_weights {                            // the tensors of a layer that owns some
+    pi_weight * w_in = nullptr;                       // latent attention: [q | dkv], lightning: [q | k | v | g] (projections of the same input, one matrix)
+    pi_weight * w_uk = nullptr, * w_uv = nullptr, * w_o = nullptr, * router = nullptr, * e_up = nullptr, * e_down = nullptr;
+    float * norm1 = nullptr, * norm2 = nullptr, * mix_norm = nullptr, * sink = nullptr, * decay = nullptr, * correction = nullptr;
+    bool loaded = false;
+};
+
 struct pi_hparams {
     pi_arch arch = PI_ARCH_LLAMA;
     int n_vocab = 0, n_ctx_train = 0, n_embd = 0, n_head = 0, n_head_kv = 0, n_layer = 0, n_ff = 0, n_rot = 0;
     float f_norm_eps = 0.0f, f_norm_rms_eps = 0.0f, rope_freq_base_train = 10000.0f, rope_freq_scale_train = 1.0f;
     float f_max_alibi_bias = 0.0f, f_clamp_kqv = 0.0f;
     pi_block block;
+    std::vector<pi_hybrid_layer> hybrid;          // PI_ARCH_FASOVIK: the layers in order
+    float embed_scale = 1.0f, residual_mult = 1.0f;
+    bool hybrid_arch() const { return arch == PI_ARCH_FASOVIK; }
+    int n_latent() const { int n = 0; for (const auto & l : hybrid) n += l.cache_index >= 0; return n; }
+    int n_recurrent() const { int n = 0; for (const auto & l : hybrid) n += l.state_index >= 0; return n; }
     int head_dim() const { return n_embd / n_head; }
     int n_embd_gqa() const { return head_dim() * n_head_kv; }
-    bool generic() const { return arch != PI_ARCH_LLAMA && arch != PI_ARCH_FALCON; }
+    bool generic() const { return arch != PI_ARCH_LLAMA && arch != PI_ARCH_FALCON && arch != PI_ARCH_FASOVIK; }
 };
 
 struct pi_layer {
@@ -65,6 +94,8 @@ struct pi_layer {
 
 struct llama_model {
     pi::gguf_file file;
+    pi::safetensors_file st_file;              // hybrid models: model.safetensors beside config.json
+    std::vector<pi_hybrid_weights> hweights;   // hybrid models: per layer (empty entries for layers that use another layer's tensors)
     pi_hparams hparams;
     pi::vocab vocab;
     std::string name, path;
@@ -85,6 +116,7 @@ struct llama_model {
     // uploads (once) token_embd if first, layers [l0,l1), final norm + output if last
     // want_mq: also make the tile-major copies of the K-quant matrices (contexts whose widest pass reaches the matrix-core kernel)
     bool ensure_loaded(int l0, int l1, bool first, bool last, bool want_mq, std::string & err);
+    bool ensure_loaded_hybrid(std::string & err);
     size_t stage_weight_bytes(int l0, int l1, bool first, bool last, int n_tok) const;
 };
 
@@ -150,6 +182,13 @@ struct llama_context {
 
     std::unique_ptr<pi::kv_cells> cells;
     uint16_t * k_cache = nullptr, * v_cache = nullptr;        // [n_layer_local][n_ctx][n_embd_gqa] f16 each
+    // hybrid models: latent cache [cells][kv_rank] fp32 per latent-attention layer (cells = the kv_cells table above), recurrent states [slots][heads][dim][vdim] fp32 per
+    // lightning layer (slots = state_slots), both at per-layer offsets into one allocation each
+    float * lat_cache = nullptr, * rec_state = nullptr; std::vector<size_t> lat_off, rec_off;
+    std::unique_ptr<pi::state_slots> slots; int n_state_slots = 8;
+    int32_t * rec_dev = nullptr;                              // per token of the pass: state slot (| 1 << 30: start from zero)
+    int exact = 0;                                            // 1: dense operators keep fp32 activations (pipeinfer_context_set_precision)
+    float * h_in = nullptr, * h_att = nullptr, * h_out = nullptr, * moe_w = nullptr, * moe_up = nullptr; int32_t * moe_sel = nullptr;   // hybrid scratch
     void * rope = nullptr;
     hipStream_t stream = nullptr;
     int stream_priority = 0;                 // > 0 high, < 0 low (pipeinfer_context_set_priority, before the first decode)

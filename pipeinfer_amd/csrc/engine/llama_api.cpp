@@ -58,7 +58,8 @@ extern "C" struct llama_context * llama_new_context_with_model(struct llama_mode
     ctx->model = model;
     ctx->cparams = params;
     ctx->n_ctx = params.n_ctx == 0 ? model->hparams.n_ctx_train : (int) params.n_ctx;       // llama.cpp:8726
-    if (ctx->n_ctx > pi_op_attention_max_cells()) {   // the attention kernel keeps a workgroup's score rows in LDS (8 rows up to 4 840 cells ... one row up to 36 200): say so HERE, not at the first decode
+    if (model->hparams.hybrid_arch() && ctx->n_ctx <= 0) { fprintf(stderr, "llama_new_context_with_model: a hybrid model needs an explicit n_ctx (its description names no training context)\n"); delete ctx; return nullptr; }
+    if (!model->hparams.hybrid_arch() && ctx->n_ctx > pi_op_attention_max_cells()) {   // the attention kernel keeps a workgroup's score rows in LDS (8 rows up to 4 840 cells ... one row up to 36 200): say so HERE, not at the first decode
         fprintf(stderr, "llama_new_context_with_model: n_ctx = %d is beyond this engine's attention kernel (one score row of n_ctx floats must fit 146 KiB of LDS: n_ctx <= %d)%s\n",
                 ctx->n_ctx, pi_op_attention_max_cells(), params.n_ctx == 0 ? "; pass an explicit n_ctx (0 selected the model's training context)" : "");
         delete ctx;
@@ -166,13 +167,40 @@ extern "C" void llama_batch_free(struct llama_batch * b) {
 // ---- KV cache API (llama.cpp:9238-9359; MPI transactions become plain host calls) --------------------------------------------
 extern "C" int  llama_get_kv_cache_token_count(const struct llama_context * ctx) { return ctx->cells->token_count(); }
 extern "C" int  llama_get_kv_cache_used_cells(const struct llama_context * ctx) { return ctx->cells->used(); }
-extern "C" void llama_kv_cache_clear(struct llama_context * ctx) { ctx->cells->clear(); }
-extern "C" void llama_kv_cache_seq_rm(struct llama_context * ctx, llama_seq_id s, llama_pos p0, llama_pos p1) { ctx->cells->seq_rm(s, p0, p1); }
+// Models with recurrent layers keep, beside the cells, ONE state per sequence (state_slots): it can be dropped, kept or copied whole, never cut — removing a range of
+// positions that is not the whole sequence is refused (the cells stay as they are, the context's error text says why).
+static bool whole_sequence(llama_pos p0, llama_pos p1) { return p0 <= 0 && p1 < 0; }
+extern "C" void llama_kv_cache_clear(struct llama_context * ctx) { ctx->cells->clear(); if (ctx->slots) ctx->slots->clear(); }
+extern "C" void llama_kv_cache_seq_rm(struct llama_context * ctx, llama_seq_id s, llama_pos p0, llama_pos p1) {
+    if (ctx->slots) {
+        if (!whole_sequence(p0, p1)) { ctx->last_error = "llama_kv_cache_seq_rm: a model with recurrent layers cannot forget part of a sequence (its state is not kept per position)"; fprintf(stderr, "%s\n", ctx->last_error.str().c_str()); return; }
+        if (s < 0) ctx->slots->clear(); else ctx->slots->release(s);
+    }
+    ctx->cells->seq_rm(s, p0, p1);
+}
 extern "C" void llama_kv_cache_seq_cp(struct llama_context * ctx, llama_seq_id a, llama_seq_id b, llama_pos p0, llama_pos p1) {
     if (a == b) return;                                                                             // llama.cpp:9296-9298
+    if (ctx->slots) {                                                                               // the destination becomes a copy of the source as it is NOW, in stream order with the runs
+        if (!whole_sequence(p0, p1)) { ctx->last_error = "llama_kv_cache_seq_cp: a model with recurrent layers copies whole sequences only"; fprintf(stderr, "%s\n", ctx->last_error.str().c_str()); return; }
+        const int src = ctx->slots->find(a);
+        if (src >= 0) {
+            const int dst = ctx->slots->acquire(b);
+            if (dst < 0) { ctx->last_error = "llama_kv_cache_seq_cp: no free state slot"; fprintf(stderr, "%s\n", ctx->last_error.str().c_str()); return; }
+            (void) ctx->slots->take_fresh(dst);
+            if (ctx->slots->is_fresh(src)) ctx->slots->mark_fresh(dst);
+            const pi_hparams & hp = ctx->model->hparams;
+            for (size_t i = 0; i < hp.hybrid.size(); i++) {
+                const pi_hybrid_layer & H = hp.hybrid[i];
+                if (H.state_index < 0) continue;
+                const size_t per = (size_t) H.heads * H.dim * H.vdim;
+                float * base = ctx->rec_state + ctx->rec_off[i];
+                if (pi_op_copy_f32(base + per * (size_t) src, base + per * (size_t) dst, (int64_t) per, ctx->stream) != 0) { ctx->last_error = std::string("llama_kv_cache_seq_cp: ") + pi_last_error(); return; }
+            }
+        }
+    }
     ctx->cells->seq_cp(a, b, p0, p1);
 }
-extern "C" void llama_kv_cache_seq_keep(struct llama_context * ctx, llama_seq_id s) { ctx->cells->seq_keep(s); }
+extern "C" void llama_kv_cache_seq_keep(struct llama_context * ctx, llama_seq_id s) { ctx->cells->seq_keep(s); if (ctx->slots) ctx->slots->keep(s); }
 extern "C" void pipeinfer_kv_cache_seq_rm_range(struct llama_context * ctx, llama_seq_id a, llama_seq_id b, llama_pos p0, llama_pos p1) { ctx->cells->seq_rm_range(a, b, p0, p1); }
 extern "C" void pipeinfer_kv_cache_seq_cp_range(struct llama_context * ctx, llama_seq_id src, llama_seq_id a, llama_seq_id b, llama_pos p0, llama_pos p1) { ctx->cells->seq_cp_range(src, a, b, p0, p1); }
 extern "C" void pipeinfer_kv_cache_seq_rm_cp_range(struct llama_context * ctx, llama_seq_id src, llama_seq_id a, llama_seq_id b, llama_pos p0, llama_pos p1) { ctx->cells->seq_rm_cp_range(src, a, b, p0, p1); }
@@ -309,6 +337,23 @@ extern "C" int pipeinfer_get_launch_rows(struct llama_context * ctx, struct pi_k
 extern "C" void pipeinfer_context_set_run_tap(struct llama_context * ctx, pipeinfer_run_tap_fn fn, void * user) { ctx->run_tap = fn; ctx->run_tap_user = user; }
 extern "C" int32_t pipeinfer_model_n_layer(const struct llama_model * model) { return model ? model->hparams.n_layer : 0; }
 extern "C" int32_t pipeinfer_run_first_cell(const struct ggml_cgraph * ticket) { return ticket ? ((const pi_run *) ticket)->kv_head : -1; }
+// dense-weight (hybrid) models: 0 = serving precision (activations rounded to bfloat16 at the matrix inputs, fp32 accumulation), 1 = every product in fp32.  Before the first decode.
+extern "C" int pipeinfer_context_set_precision(struct llama_context * ctx, int exact) {
+    if (!ctx->model->hparams.hybrid_arch()) { ctx->last_error = "pipeinfer_context_set_precision: GGUF models compute as their quantisation types prescribe"; return -1; }
+    if (!ctx->inflight.empty()) { ctx->last_error = "pipeinfer_context_set_precision: runs are in flight"; return -1; }
+    if ((exact != 0) != (ctx->exact != 0)) { std::lock_guard<std::mutex> lk(ctx->graphs_mu); for (auto & kv : ctx->graphs) if (kv.second.exec) { (void) hipGraphExecDestroy(kv.second.exec); kv.second.exec = nullptr; } }
+    ctx->exact = exact != 0;
+    return 0;
+}
+// models with recurrent layers: how many sequences can be live at once (one state slot each).  Before the first decode.
+extern "C" int pipeinfer_context_set_state_slots(struct llama_context * ctx, int n_slots) {
+    if (ctx->prepared) { ctx->last_error = "pipeinfer_context_set_state_slots: the context has already decoded"; return -1; }
+    if (n_slots < 1) { ctx->last_error = "pipeinfer_context_set_state_slots: at least one slot"; return -1; }
+    ctx->n_state_slots = n_slots;
+    return 0;
+}
+extern "C" int pipeinfer_get_state_slots_used(struct llama_context * ctx) { return ctx->slots ? ctx->slots->used() : 0; }
+
 extern "C" void pipeinfer_context_set_graphs(struct llama_context * ctx, int enable) { ctx->use_graphs = enable != 0 && getenv("PI_NO_GRAPHS") == nullptr; }
 
 extern "C" void pipeinfer_context_set_remote(struct llama_context * ctx, const struct pipeinfer_remote_ops * ops) {

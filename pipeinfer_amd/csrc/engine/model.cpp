@@ -2,6 +2,7 @@
 // (tensor names/shapes: llama.cpp:2756-2824 Llama, :2891-2968 Falcon).
 #include "engine.h"
 
+#include <algorithm>
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -38,6 +39,7 @@ llama_model::~llama_model() {
         pi_weight_free(l.wq); pi_weight_free(l.wk); pi_weight_free(l.wv); pi_weight_free(l.wo); pi_weight_free(l.wqkv);
         pi_weight_free(l.ffn_gate); pi_weight_free(l.ffn_down); pi_weight_free(l.ffn_up);
     }
+    for (auto & w : hweights) { pi_weight_free(w.w_in); pi_weight_free(w.w_uk); pi_weight_free(w.w_uv); pi_weight_free(w.w_o); pi_weight_free(w.router); pi_weight_free(w.e_up); pi_weight_free(w.e_down); }
     pi_weight_free(tok_embd); pi_weight_free(output); pi_weight_free(pos_embd);
     for (void * p : f32_allocs) pi_free(p);
 }
@@ -180,6 +182,16 @@ bool llama_model::ensure_loaded(int l0, int l1, bool first, bool last, bool want
 // sum of ggml_nbytes of the tensors one decode call on this stage streams: the embedding contributes n_tok rows
 size_t llama_model::stage_weight_bytes(int l0, int l1, bool first, bool last, int n_tok) const {
     size_t b = 0;
+    if (hparams.hybrid_arch()) {                                              // every layer's matrices and vectors once, the experts a token does not choose left out, + the embedding rows
+        for (size_t i = 0; i < hparams.hybrid.size(); i++) {
+            const pi_hybrid_layer & H = hparams.hybrid[i];
+            const size_t w = (size_t) hparams.n_embd;
+            b += 2 * (size_t) H.in_rows() * w + 2 * (size_t) H.heads * H.vdim * w + 4 * w;
+            if (H.mixer == PI_MIXER_LATENT_ATTENTION) b += 2 * (size_t) H.kv_rank * H.heads * (H.dim + H.vdim);
+            if (H.has_mlp) b += 2 * (size_t) (H.n_expert + H.n_identity) * w + (size_t) std::min(H.n_expert, std::max(1, n_tok) * H.top) * 4 * (size_t) H.ff * w;
+        }
+        return b + 2 * (size_t) hparams.n_vocab * hparams.n_embd + 2 * (size_t) n_tok * hparams.n_embd;
+    }
     auto add = [&](const std::string & name, int64_t rows_used) {
         const pi::gguf_tensor * t = file.tensor(name);
         if (t) b += rows_used < 0 ? t->nbytes : pi::type_row_size(t->type, t->ne[0]) * (size_t) rows_used;
@@ -194,7 +206,13 @@ size_t llama_model::stage_weight_bytes(int l0, int l1, bool first, bool last, in
     return b;
 }
 
+namespace pi { bool is_hybrid_model_path(const std::string & path, std::string & folder); llama_model * load_hybrid_model(const std::string & folder, const llama_model_params & params); }
+
 extern "C" struct llama_model * llama_load_model_from_file(const char * path, struct llama_model_params params) {
+    {   // a folder (config.json + model.safetensors) instead of a GGUF file: the hybrid architectures (model_hybrid.cpp)
+        std::string folder;
+        if (pi::is_hybrid_model_path(path, folder)) return pi::load_hybrid_model(folder, params);
+    }
     std::unique_ptr<llama_model> m(new llama_model());
     std::string err;
     m->path = path;
@@ -280,7 +298,7 @@ extern "C" enum llama_vocab_type llama_vocab_type(const struct llama_model * m) 
 extern "C" uint64_t llama_model_size(const struct llama_model * m) { return m->n_bytes; }
 extern "C" uint64_t llama_model_n_params(const struct llama_model * m) { return m->n_elements; }
 extern "C" int llama_model_desc(const struct llama_model * m, char * buf, size_t n) {
-    static const char * names[] = { "llama", "falcon", "baichuan", "starcoder", "refact", "bloom", "mpt", "stablelm", "persimmon" };
+    static const char * names[] = { "llama", "falcon", "baichuan", "starcoder", "refact", "bloom", "mpt", "stablelm", "persimmon", "fasovik" };
     return snprintf(buf, n, "%s %s", names[m->hparams.arch], m->name.c_str());
 }
 

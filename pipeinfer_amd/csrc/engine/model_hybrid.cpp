@@ -1,0 +1,209 @@
+// Hybrid models described by a folder: config.json (the layer list with every size and constant) + model.safetensors (bfloat16 tensors, linear weights [out][in]).
+//
+// config.json:  architecture, vocab, width, embedding.scale, norm.eps, residual_mult, layers[]: { type: "latent_attention" | "lightning", mixer: { heads, dim, vdim,
+// kv_rank + scale | decay[] }, mlp: null | { kind: "moe", expert.ff, router.experts / identity / top }, weights_of: j (optional: the layer has no tensors, it uses layer j's) }.
+// Tensors: embed, final.norm, l<i>.norm1 / norm2, l<i>.mix.{q, dkv, dkv.norm, uk, uv, sink, o} or l<i>.mix.{q, k, v, g, o, norm}, l<i>.mlp.{router, correction, e<k>.up, e<k>.down}.
+// Projections that read the same input are uploaded as ONE matrix (rows one after the other) so that they are one launch; vectors go up as fp32.
+#include "engine.h"
+#include "json.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <sstream>
+#include <sys/stat.h>
+
+namespace {
+
+bool num_at(const pi::json & j, const char * path, double & out) { const pi::json * v = j.at(path); if (!v || !v->is_num()) return false; out = v->num; return true; }
+bool int_at(const pi::json & j, const char * path, int & out) { double d; if (!num_at(j, path, d) || d != std::floor(d) || d < 0 || d > 1e9) return false; out = (int) d; return true; }
+
+float bf16_to_f32(uint16_t b) { const uint32_t u = (uint32_t) b << 16; float f; memcpy(&f, &u, 4); return f; }
+
+struct loader {
+    llama_model & m; std::string & err;
+    const pi::st_tensor * get(const std::string & name, std::initializer_list<int64_t> shape) {
+        const pi::st_tensor * t = m.st_file.tensor(name);
+        if (!t) { err = "missing tensor " + name; return nullptr; }
+        if (t->dtype != "BF16") { err = "tensor " + name + " is " + t->dtype + ", expected BF16"; return nullptr; }
+        if (t->shape != std::vector<int64_t>(shape)) {
+            std::string got, want;
+            for (int64_t d : t->shape) got += (got.empty() ? "" : ",") + std::to_string(d);
+            for (int64_t d : shape) want += (want.empty() ? "" : ",") + std::to_string(d);
+            err = "tensor " + name + " has shape [" + got + "], expected [" + want + "]"; return nullptr;
+        }
+        return t;
+    }
+    // rows of several [rows_i][k] tensors one after the other as one bfloat16 matrix
+    pi_weight * matrix(const std::vector<std::pair<std::string, int64_t>> & parts, int64_t k) {
+        std::vector<uint16_t> host; int64_t rows = 0;
+        const uint8_t * single = nullptr;
+        for (const auto & p : parts) {
+            const pi::st_tensor * t = get(p.first, { p.second, k });
+            if (!t) return nullptr;
+            if (parts.size() == 1) single = t->data;
+            else { const size_t at = host.size(); host.resize(at + (size_t) p.second * k); memcpy(host.data() + at, t->data, t->nbytes); }
+            rows += p.second;
+        }
+        pi_weight * w = pi_weight_upload(PI_BF16, k, rows, single ? (const void *) single : (const void *) host.data(), nullptr);
+        if (!w) { err = "upload of " + parts[0].first + " failed: " + pi_last_error(); return nullptr; }
+        m.hbm_bytes += pi_weight_nbytes(w);
+        m.matrices.push_back({ w, nullptr, -1 });
+        return w;
+    }
+    float * vector_f32(const std::vector<float> & v) {
+        float * d = (float *) pi_malloc(std::max<size_t>(v.size(), 1) * 4);
+        if (!d || (!v.empty() && (pi_memcpy_h2d(d, v.data(), v.size() * 4, nullptr) || pi_stream_sync(nullptr)))) { err = std::string("upload of a vector failed: ") + pi_last_error(); return nullptr; }
+        m.f32_allocs.push_back(d); m.hbm_bytes += v.size() * 4;
+        return d;
+    }
+    float * vector(const std::string & name, int64_t n) {
+        const pi::st_tensor * t = get(name, { n });
+        if (!t) return nullptr;
+        std::vector<float> v((size_t) n);
+        for (int64_t i = 0; i < n; i++) v[(size_t) i] = bf16_to_f32(((const uint16_t *) t->data)[i]);
+        return vector_f32(v);
+    }
+};
+
+}  // namespace
+
+bool llama_model::ensure_loaded_hybrid(std::string & err) {
+    const pi_hparams & hp = hparams;
+    loader L{ *this, err };
+    pi_weight_set_mq_copies(0);
+    struct restore { ~restore() { pi_weight_set_mq_copies(1); } } r;
+    const int64_t width = hp.n_embd;
+    if (!tok_embd) {
+        if (!(tok_embd = L.matrix({ { "embed", hp.n_vocab } }, width))) return false;
+        if (!(output_norm = L.vector("final.norm", width))) return false;
+    }
+    for (size_t i = 0; i < hp.hybrid.size(); i++) {
+        const pi_hybrid_layer & H = hp.hybrid[i];
+        pi_hybrid_weights & W = hweights[i];
+        if (H.weights != (int) i || W.loaded) continue;
+        const std::string p = "l" + std::to_string(i) + ".";
+        const int64_t hd = (int64_t) H.heads * H.dim, hv = (int64_t) H.heads * H.vdim;
+        if (!(W.norm1 = L.vector(p + "norm1", width))) return false;
+        if (H.mixer == PI_MIXER_LIGHTNING) {
+            if (!(W.w_in = L.matrix({ { p + "mix.q", hd }, { p + "mix.k", hd }, { p + "mix.v", hv }, { p + "mix.g", hv } }, width))) return false;
+            if (!(W.mix_norm = L.vector(p + "mix.norm", hv))) return false;
+            if (!(W.decay = L.vector_f32(H.decay))) return false;
+        } else {
+            if (!(W.w_in = L.matrix({ { p + "mix.q", hd }, { p + "mix.dkv", H.kv_rank } }, width))) return false;
+            if (!(W.mix_norm = L.vector(p + "mix.dkv.norm", H.kv_rank))) return false;
+            if (!(W.w_uk = L.matrix({ { p + "mix.uk", hd } }, H.kv_rank)) || !(W.w_uv = L.matrix({ { p + "mix.uv", hv } }, H.kv_rank))) return false;
+            if (!(W.sink = L.vector(p + "mix.sink", H.heads))) return false;
+        }
+        if (!(W.w_o = L.matrix({ { p + "mix.o", width } }, hv))) return false;
+        if (H.has_mlp) {
+            if (!(W.norm2 = L.vector(p + "norm2", width))) return false;
+            const int n_out = H.n_expert + H.n_identity;
+            if (!(W.router = L.matrix({ { p + "mlp.router", n_out } }, width)) || !(W.correction = L.vector(p + "mlp.correction", n_out))) return false;
+            if (H.n_expert > 0) {
+                std::vector<std::pair<std::string, int64_t>> ups, downs;
+                for (int e = 0; e < H.n_expert; e++) { ups.push_back({ p + "mlp.e" + std::to_string(e) + ".up", H.ff }); downs.push_back({ p + "mlp.e" + std::to_string(e) + ".down", width }); }
+                if (!(W.e_up = L.matrix(ups, width)) || !(W.e_down = L.matrix(downs, H.ff))) return false;
+            }
+        }
+        W.loaded = true;
+    }
+    return true;
+}
+
+namespace pi {
+
+// path: the folder, or its config.json / model.safetensors
+bool is_hybrid_model_path(const std::string & path, std::string & folder) {
+    struct stat st;
+    if (stat(path.c_str(), &st) != 0) return false;
+    if (S_ISDIR(st.st_mode)) { folder = path; return stat((path + "/config.json").c_str(), &st) == 0; }
+    const size_t slash = path.find_last_of('/');
+    const std::string base = slash == std::string::npos ? path : path.substr(slash + 1);
+    if (base != "config.json" && base != "model.safetensors") return false;
+    folder = slash == std::string::npos ? "." : path.substr(0, slash);
+    return true;
+}
+
+llama_model * load_hybrid_model(const std::string & folder, const llama_model_params & params) {
+    std::unique_ptr<llama_model> m(new llama_model());
+    m->path = folder; m->device = params.main_gpu;
+    auto fail = [&](const std::string & what) { fprintf(stderr, "llama_load_model_from_file: %s/config.json: %s\n", folder.c_str(), what.c_str()); return (llama_model *) nullptr; };
+    std::ifstream in(folder + "/config.json");
+    if (!in) return fail("cannot be read");
+    std::stringstream ss; ss << in.rdbuf();
+    json cfg; std::string err;
+    if (!json::parse(ss.str(), cfg, err) || !cfg.is_obj()) return fail(err.empty() ? "not a JSON object" : err);
+    const json * arch = cfg.find("architecture");
+    if (!arch || !arch->is_str()) return fail("no 'architecture'");
+    pi_hparams & hp = m->hparams;
+    // the registry of folder-described architectures (GGUF files name theirs in general.architecture, model.cpp)
+    if (arch->str == "Fasovik") hp.arch = PI_ARCH_FASOVIK;
+    else return fail("architecture '" + arch->str + "' is not one this engine builds (Fasovik)");
+    m->name = arch->str;
+    double d;
+    if (!int_at(cfg, "vocab", hp.n_vocab) || !int_at(cfg, "width", hp.n_embd) || hp.n_vocab < 1 || hp.n_embd < 1) return fail("'vocab' and 'width' must be positive integers");
+    if (!num_at(cfg, "embedding.scale", d)) return fail("no 'embedding.scale'");
+    hp.embed_scale = (float) d;
+    if (!num_at(cfg, "norm.eps", d)) return fail("no 'norm.eps'");
+    hp.f_norm_rms_eps = (float) d;
+    if (!num_at(cfg, "residual_mult", d)) return fail("no 'residual_mult'");
+    hp.residual_mult = (float) d;
+    const json * layers = cfg.find("layers");
+    if (!layers || !layers->is_arr() || layers->arr.empty()) return fail("'layers' must be a non-empty list");
+    hp.n_layer = (int) layers->arr.size();
+    hp.n_head = hp.n_head_kv = 1; hp.n_ctx_train = 0;
+    int n_cache = 0, n_state = 0;
+    for (int i = 0; i < hp.n_layer; i++) {
+        const json & jl = layers->arr[(size_t) i];
+        const std::string where = "layers[" + std::to_string(i) + "]: ";
+        pi_hybrid_layer H;
+        const json * type = jl.find("type");
+        if (!type || !type->is_str()) return fail(where + "no 'type'");
+        if (type->str == "latent_attention") H.mixer = PI_MIXER_LATENT_ATTENTION;
+        else if (type->str == "lightning") H.mixer = PI_MIXER_LIGHTNING;
+        else return fail(where + "mixer type '" + type->str + "' is unknown (latent_attention, lightning)");
+        if (!int_at(jl, "mixer.heads", H.heads) || !int_at(jl, "mixer.dim", H.dim) || !int_at(jl, "mixer.vdim", H.vdim) || H.heads < 1 || H.dim < 1 || H.vdim < 1) return fail(where + "mixer needs positive 'heads', 'dim', 'vdim'");
+        if (H.mixer == PI_MIXER_LATENT_ATTENTION) {
+            if (!int_at(jl, "mixer.kv_rank", H.kv_rank) || H.kv_rank < 1 || !num_at(jl, "mixer.scale", d)) return fail(where + "latent_attention needs 'kv_rank' and 'scale'");
+            H.scale = (float) d;
+            H.cache_index = n_cache++;
+        } else {
+            const json * dec = jl.at("mixer.decay");
+            if (!dec || !dec->is_arr() || (int) dec->arr.size() != H.heads) return fail(where + "lightning needs 'decay' with one value per head");
+            for (const json & v : dec->arr) { if (!v.is_num()) return fail(where + "'decay' holds a non-number"); H.decay.push_back((float) v.num); }
+            if (H.dim > 1024) return fail(where + "lightning key width above 1024");
+            H.state_index = n_state++;
+        }
+        H.weights = i;
+        if (jl.has("weights_of")) {
+            if (!int_at(jl, "weights_of", H.weights) || H.weights >= hp.n_layer) return fail(where + "'weights_of' names no layer");
+        }
+        if (jl.has("mlp")) {
+            const json * kind = jl.at("mlp.kind");
+            if (!kind || !kind->is_str() || kind->str != "moe") return fail(where + "feed-forward kind must be 'moe'");
+            if (!int_at(jl, "mlp.router.experts", H.n_expert) || !int_at(jl, "mlp.router.identity", H.n_identity) || !int_at(jl, "mlp.router.top", H.top)) return fail(where + "mlp.router needs 'experts', 'identity', 'top'");
+            if (H.n_expert > 0 && (!int_at(jl, "mlp.expert.ff", H.ff) || H.ff < 1)) return fail(where + "mlp.expert needs 'ff'");
+            if (H.top < 1 || H.top > H.n_expert + H.n_identity) return fail(where + "'top' must lie between 1 and the number of router outputs");
+            H.has_mlp = true;
+        }
+        hp.hybrid.push_back(std::move(H));
+    }
+    for (int i = 0; i < hp.n_layer; i++) {                                   // a layer that borrows tensors must be the same kind of layer with the same sizes
+        const pi_hybrid_layer & a = hp.hybrid[(size_t) i], & b = hp.hybrid[(size_t) a.weights];
+        if (b.weights != a.weights) return fail("layers[" + std::to_string(i) + "]: 'weights_of' names a layer that has no tensors of its own");
+        if (a.mixer != b.mixer || a.heads != b.heads || a.dim != b.dim || a.vdim != b.vdim || a.kv_rank != b.kv_rank || a.has_mlp != b.has_mlp || a.n_expert != b.n_expert || a.n_identity != b.n_identity || a.ff != b.ff)
+            return fail("layers[" + std::to_string(i) + "]: its sizes differ from those of the layer whose tensors it uses");
+    }
+    m->hweights.resize((size_t) hp.n_layer);
+    if (!params.vocab_only) {
+        if (!m->st_file.open(folder + "/model.safetensors", err)) { fprintf(stderr, "llama_load_model_from_file: %s\n", err.c_str()); return nullptr; }
+        for (const auto & kv : m->st_file.tensors) { m->n_elements += (uint64_t) kv.second.elements(); m->n_bytes += kv.second.nbytes; }
+        const st_tensor * e = m->st_file.tensor("embed");
+        if (!e || e->shape != std::vector<int64_t>{ hp.n_vocab, hp.n_embd }) return fail("tensor 'embed' is missing or not [vocab][width]");
+    }
+    return m.release();
+}
+
+}  // namespace pi

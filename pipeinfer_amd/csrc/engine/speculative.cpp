@@ -700,6 +700,9 @@ extern "C" int pipeinfer_speculative(struct llama_context * ctx_tgt, struct llam
                                      const llama_token * prompt, int32_t n_prompt, llama_token * out_tokens, int32_t out_cap, struct pipeinfer_spec_result * result) {
     driver d;
     d.tgt = ctx_tgt; d.dft = ctx_dft; d.P = *params;
+    if (ctx_tgt->model->hparams.n_recurrent() > 0 || (ctx_dft && ctx_dft->model->hparams.n_recurrent() > 0)) {
+        fprintf(stderr, "pipeinfer_speculative: a model with recurrent layers cannot take back rejected tokens (one state per sequence, not one cell per position): generate it with llama_decode\n"); return -1;
+    }
     if (params->mode < 0 || params->mode > 2) { fprintf(stderr, "pipeinfer_speculative: unknown mode %d\n", params->mode); return -1; }
     if (!ctx_tgt->cparams.logits_all || (params->mode != 2 && !ctx_dft->cparams.logits_all)) { fprintf(stderr, "pipeinfer_speculative: both contexts need logits_all (speculative.cpp:115)\n"); return -1; }
     ctx_tgt->canceled_batches.clear();                       // batch ids restart at 1 for every call

@@ -73,11 +73,11 @@ int pi_mmq_step(int type, int n_tok, int64_t rows);             // tokens per ma
 
 static inline bool pi_type_is_legacy(int t) { return t == PI_Q4_1 || t == PI_Q5_0 || t == PI_Q5_1; }
 static inline int pi_type_blck(int t) {
-    switch (t) { case PI_F32: case PI_F16: return 1; case PI_Q4_0: case PI_Q4_1: case PI_Q5_0: case PI_Q5_1: case PI_Q8_0: case PI_Q8_1: return 32; default: return 256; }
+    switch (t) { case PI_F32: case PI_F16: case PI_BF16: return 1; case PI_Q4_0: case PI_Q4_1: case PI_Q5_0: case PI_Q5_1: case PI_Q8_0: case PI_Q8_1: return 32; default: return 256; }
 }
 static inline int pi_type_size(int t) {
     switch (t) {
-        case PI_F32: return 4; case PI_F16: return 2; case PI_Q4_0: return 18; case PI_Q8_0: return 34;
+        case PI_F32: return 4; case PI_F16: case PI_BF16: return 2; case PI_Q4_0: return 18; case PI_Q8_0: return 34;
         case PI_Q4_1: return 20; case PI_Q5_0: return 22; case PI_Q5_1: return 24; case PI_Q8_1: return 40;
         case PI_Q2_K: return 84; case PI_Q3_K: return 110; case PI_Q4_K: return 144; case PI_Q5_K: return 176; case PI_Q6_K: return 210; case PI_Q8_K: return 292;
     }

@@ -450,7 +450,7 @@ extern "C" pi_weight * pi_weight_upload(int type, int64_t ne0, int64_t ne1, cons
     uint8_t * base = (uint8_t *) w->base;
     w->p0 = base; w->p1 = w->p2 = w->p3 = nullptr; w->mq = nullptr; w->mq_base = nullptr;
     auto fail = [&](const char * what) { pi_set_error("pi_weight_upload: %s", what); (void) hipFree(w->base); delete w; return (pi_weight *) nullptr; };
-    if (type == PI_F32 || type == PI_F16) {
+    if (type == PI_F32 || type == PI_F16 || type == PI_BF16) {
         if (hipMemcpyAsync(base, host, w->nbytes, hipMemcpyHostToDevice, stream) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) return fail("H2D copy failed");
         return w;
     }

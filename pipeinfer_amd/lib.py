@@ -126,3 +126,13 @@ def _declare(lib):
     lib.pi_op_add.argtypes = [vp, vp, vp, i64, vp]
     lib.pi_op_topk_scratch_bytes.argtypes = [i32]; lib.pi_op_topk_scratch_bytes.restype = C.c_size_t
     lib.pi_op_topk.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, vp]
+    # dense bfloat16 matrices and the operators of hybrid blocks
+    lib.pi_op_embed.argtypes = [vp, vp, i32, f32, vp, vp]
+    lib.pi_op_dense.argtypes = [vp, vp, i64, i32, vp, i64, i32, i64, i32, i32, vp]
+    lib.pi_op_rms_scale.argtypes = [vp, i64, vp, f32, f32, i32, i32, vp, i64, vp, i64, f32, vp, i64, vp, i32, vp]
+    lib.pi_op_linear_attention.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp, vp, vp, i32, i32, vp, i64, vp]
+    lib.pi_op_copy_f32.argtypes = [vp, vp, i64, vp]
+    lib.pi_op_latent_attention.argtypes = [vp, i64, vp, vp, vp, vp, vp, f32, i32, i32, i32, i32, i32, i32, vp, i64, vp, vp]
+    lib.pi_op_latent_attention_max_cells.argtypes = [i32]
+    lib.pi_op_moe_route.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp, vp, vp]
+    lib.pi_op_moe_experts.argtypes = [vp, vp, i32, i32, vp, i64, vp, vp, i32, i32, i32, vp, vp, i64, vp]

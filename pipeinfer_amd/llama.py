@@ -195,6 +195,7 @@ class Context:
         if not self.h:
             raise L.PipeInferError("llama_new_context_with_model failed")
         self.n_vocab = model.n_vocab
+        self.n_batch = n_batch
 
     def set_priority(self, priority):
         self.lib.pipeinfer_context_set_priority.argtypes = [C.c_void_p, C.c_int]
@@ -230,6 +231,22 @@ class Context:
         self.lib.pipeinfer_context_set_run_tap.restype = None
         self.lib.pipeinfer_context_set_run_tap(self.h, C.cast(self._tap, C.c_void_p) if fn else None, None)
 
+    def set_precision(self, exact):
+        """hybrid (safetensors) models: False = serving precision (bfloat16 matrix inputs, fp32 accumulation), True = every product in fp32"""
+        self.lib.pipeinfer_context_set_precision.argtypes = [C.c_void_p, C.c_int]
+        if self.lib.pipeinfer_context_set_precision(self.h, int(bool(exact))) != 0:
+            raise L.PipeInferError(self.lib.pipeinfer_context_error(self.h).decode())
+
+    def set_state_slots(self, n):
+        """models with recurrent layers: sequences that can be live at once"""
+        self.lib.pipeinfer_context_set_state_slots.argtypes = [C.c_void_p, C.c_int]
+        if self.lib.pipeinfer_context_set_state_slots(self.h, int(n)) != 0:
+            raise L.PipeInferError(self.lib.pipeinfer_context_error(self.h).decode())
+
+    def state_slots_used(self):
+        self.lib.pipeinfer_get_state_slots_used.argtypes = [C.c_void_p]
+        return int(self.lib.pipeinfer_get_state_slots_used(self.h))
+
     def set_graphs(self, enable):
         self.lib.pipeinfer_context_set_graphs.argtypes = [C.c_void_p, C.c_int]
         self.lib.pipeinfer_context_set_graphs.restype = None
@@ -245,6 +262,25 @@ class Context:
         if rc != 0:
             raise L.PipeInferError(f"llama_decode rc={rc}: {self.lib.pipeinfer_context_error(self.h).decode()}")
         return self.logits(len(tokens))
+
+    def feed(self, tokens, pos0, seq=0):
+        """the next tokens of ONE sequence from position pos0 on, in passes of at most n_batch tokens (what a generation loop does with a long prompt); logits of every token"""
+        out = []
+        for a in range(0, len(tokens), self.n_batch):
+            part = list(tokens[a:a + self.n_batch])
+            out.append(self.decode(part, [pos0 + a + i for i in range(len(part))], [[seq]] * len(part)))
+        return np.concatenate(out) if out else np.zeros((0, self.n_vocab), np.float32)
+
+    def generate(self, prompt, n_predict, seq=0, pos0=0):
+        """greedy continuation of one sequence through llama_decode and the engine's device-side top-k (the arg-max llama_sample_token_greedy takes)"""
+        self.feed(prompt[:-1], pos0, seq)
+        out, last, pos = [], prompt[-1], pos0 + len(prompt) - 1
+        for _ in range(n_predict):
+            self.decode([last], [pos], [[seq]])
+            last = self.topk(0)[0][0]
+            out.append(last)
+            pos += 1
+        return out
 
     def start(self, tokens, pos, seq_ids, batch_id=0):
         b = Batch(tokens, pos, seq_ids, batch_id)

@@ -44,6 +44,16 @@ LLAMA_API int  pipeinfer_context_set_coalescing(struct llama_context * ctx, int 
 LLAMA_API int pipeinfer_context_set_precision(struct llama_context * ctx, int exact);
 LLAMA_API int pipeinfer_context_set_state_slots(struct llama_context * ctx, int n_slots);
 LLAMA_API int pipeinfer_get_state_slots_used(struct llama_context * ctx);
+/* the slot table on its own (host only): acquire = the sequence's slot, allotted now if it has none (-1: all taken); take_fresh = 1 once per allotment (the state starts from zero) */
+LLAMA_API void * pi_stateslots_new(int n_slots);
+LLAMA_API void pi_stateslots_free(void * slots);
+LLAMA_API int pi_stateslots_acquire(void * slots, int seq);
+LLAMA_API int pi_stateslots_take_fresh(void * slots, int slot);
+LLAMA_API int pi_stateslots_find(void * slots, int seq);
+LLAMA_API int pi_stateslots_used(void * slots);
+LLAMA_API void pi_stateslots_release(void * slots, int seq);
+LLAMA_API void pi_stateslots_keep(void * slots, int seq);
+LLAMA_API void pi_stateslots_clear(void * slots);
 LLAMA_API void pipeinfer_context_set_graphs(struct llama_context * ctx, int enable);
 LLAMA_API const char * pipeinfer_context_error(struct llama_context * ctx);
 LLAMA_API int32_t pipeinfer_model_n_layer(const struct llama_model * model);

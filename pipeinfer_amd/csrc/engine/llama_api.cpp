@@ -354,6 +354,17 @@ extern "C" int pipeinfer_context_set_state_slots(struct llama_context * ctx, int
 }
 extern "C" int pipeinfer_get_state_slots_used(struct llama_context * ctx) { return ctx->slots ? ctx->slots->used() : 0; }
 
+// stand-alone state-slot table (tests: the bookkeeping without a GPU)
+extern "C" void * pi_stateslots_new(int n) { return new pi::state_slots(n); }
+extern "C" void pi_stateslots_free(void * s) { delete (pi::state_slots *) s; }
+extern "C" int pi_stateslots_acquire(void * s, int seq) { return ((pi::state_slots *) s)->acquire(seq); }
+extern "C" int pi_stateslots_take_fresh(void * s, int slot) { return ((pi::state_slots *) s)->take_fresh(slot) ? 1 : 0; }
+extern "C" int pi_stateslots_find(void * s, int seq) { return ((pi::state_slots *) s)->find(seq); }
+extern "C" int pi_stateslots_used(void * s) { return ((pi::state_slots *) s)->used(); }
+extern "C" void pi_stateslots_release(void * s, int seq) { ((pi::state_slots *) s)->release(seq); }
+extern "C" void pi_stateslots_keep(void * s, int seq) { ((pi::state_slots *) s)->keep(seq); }
+extern "C" void pi_stateslots_clear(void * s) { ((pi::state_slots *) s)->clear(); }
+
 extern "C" void pipeinfer_context_set_graphs(struct llama_context * ctx, int enable) { ctx->use_graphs = enable != 0 && getenv("PI_NO_GRAPHS") == nullptr; }
 
 extern "C" void pipeinfer_context_set_remote(struct llama_context * ctx, const struct pipeinfer_remote_ops * ops) {

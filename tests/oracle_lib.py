@@ -108,7 +108,7 @@ def ref_kv():
     if _ref_kv is None:
         path = os.path.join(ORACLE_DIR, "_ref", "libref_kv.so")
         if not os.path.exists(path):
-            if os.path.isdir("/root/reference"):
+            if os.path.exists("/root/reference/ggml.c"):
                 subprocess.check_call(["make", "-C", ORACLE_DIR, "ref"], stdout=subprocess.DEVNULL)
             else:
                 return None
@@ -146,7 +146,7 @@ def ref():
     global _ref
     if _ref is None:
         if not have_ref():
-            if os.path.isdir("/root/reference"):
+            if os.path.exists("/root/reference/ggml.c"):
                 subprocess.check_call(["make", "-C", ORACLE_DIR, "ref"], stdout=subprocess.DEVNULL)
             else:
                 return None

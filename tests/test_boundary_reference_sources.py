@@ -18,7 +18,7 @@ from pipeinfer_amd import lib as L
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 REF = "/root/reference"
 LIBDIR = os.path.join(ROOT, "pipeinfer_amd")
-need_ref = pytest.mark.skipif(not os.path.isdir(REF) or shutil.which("g++") is None, reason="needs the reference sources and a host compiler")
+need_ref = pytest.mark.skipif(not os.path.exists(os.path.join(REF, "ggml.c")) or shutil.which("g++") is None, reason="needs the reference sources and a host compiler")
 
 
 @need_ref
@@ -51,7 +51,7 @@ def test_boundary_struct_layouts_are_compile_time_checked():
     assert "static_assert(sizeof(llama_batch) == 80" in text and "offsetof(llama_batch, batch_id) == 68" in text
     r = subprocess.run(["g++", "-std=c++11", "-fsyntax-only", "-I" + os.path.join(ROOT, "include"), src], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr[-3000:]
-    if os.path.isdir(REF):
+    if os.path.exists(os.path.join(REF, "llama.h")):
         asserts = text[text.index("static_assert(sizeof(llama_batch)"):text.index("static void batch_add")]
         probe = "#include <cstddef>\n" + asserts
         r = subprocess.run(["g++", "-std=c++11", "-fsyntax-only", "-I" + REF, "-include", os.path.join(REF, "llama.h"), "-x", "c++", "-"], input=probe, capture_output=True, text=True, timeout=120)

@@ -488,7 +488,13 @@ def main():
     ap.add_argument("--adaptive-pause", type=int, default=0)
     ap.add_argument("--detail", default=os.environ.get("PIPEINFER_BENCH_DETAIL", "/tmp/pipeinfer_bench_detail.json"),
                     help="where the full result (per-instance table, every family, cancel / segment statistics) is written; the stdout line stays small")
+    ap.add_argument("--compare-hybrid", nargs="?", const="w1024,w2048,w4096", default=None, metavar="SIZES",
+                    help="instead of the default workload: prefill / decode throughput and per-kernel roofline fractions of the Fasovik design at these layer sizes beside a Llama "
+                         "model of equal size (pipeinfer_amd/tools/hybrid_bench.py); one JSON line per size")
     args = ap.parse_args()
+    if args.compare_hybrid:
+        from pipeinfer_amd.tools import hybrid_bench
+        return hybrid_bench.main(args.compare_hybrid.split(","), args.cache)
 
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         # started as ONE command (the reference starts every rank from one mpirun: ggml-mpi.c:58-61 MPI_Init_thread, speculative.cpp:116-139 comm split):

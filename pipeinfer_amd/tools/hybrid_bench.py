@@ -1,0 +1,155 @@
+"""Prefill and decode throughput of the Fasovik design at layer sizes of real models (random weights), beside the engine's closest GGUF model — a Llama-architecture model of the
+same width, depth and head count with Q8_0 weights, the densest quantised type the mat-vec kernels take — and the kernels' distance from the roofline for both.
+
+`bench.py --compare-hybrid [SIZE,...]` prints one JSON line per size; bench.py's default workload and line are untouched."""
+import ctypes as C
+import json
+import os
+import struct
+import sys
+import time
+
+import numpy as np
+
+from .. import lib as L, llama as LL
+from . import synth
+
+HBM_PEAK = 8.0e12
+BF16_PEAK = 2.5e15
+
+# name -> width, layers, heads, dim, vdim, kv_rank, experts, identity, top, ff, vocab
+SIZES = {
+    "w1024": (1024, 4, 16, 64, 64, 256, 8, 2, 2, 512, 32000),
+    "w2048": (2048, 4, 16, 128, 128, 512, 8, 2, 2, 1024, 32000),
+    "w4096": (4096, 2, 32, 128, 128, 512, 8, 2, 2, 2048, 32000),
+}
+FAMILIES = {0: "matvec", 1: "matrix_cores", 2: "norm_quant", 3: "quant", 4: "act_quant", 5: "attention", 6: "other"}
+
+
+def write_fasovik(folder, size, seed=1):
+    width, n_layer, heads, dim, vdim, rank, n_exp, n_id, top, ff, vocab = SIZES[size]
+    layers = []
+    for i in range(n_layer):
+        mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": n_exp, "identity": n_id, "top": top}}
+        if i % 2 == 0:
+            layers.append({"type": "latent_attention", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": rank, "scale": dim ** -0.5}, "mlp": mlp})
+        else:
+            layers.append({"type": "lightning", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "decay": [float(1.0 - 2.0 ** (-3 - 5 * h / heads)) for h in range(heads)]}, "mlp": mlp})
+    cfg = {"architecture": "Fasovik", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": layers}
+    shapes = {"embed": (vocab, width), "final.norm": (width,)}
+    for i, l in enumerate(layers):
+        p = "l%d." % i
+        shapes[p + "norm1"] = shapes[p + "norm2"] = (width,)
+        hd, hv = heads * dim, heads * vdim
+        if l["type"] == "lightning":
+            shapes.update({p + "mix.q": (hd, width), p + "mix.k": (hd, width), p + "mix.v": (hv, width), p + "mix.g": (hv, width), p + "mix.o": (width, hv), p + "mix.norm": (hv,)})
+        else:
+            shapes.update({p + "mix.q": (hd, width), p + "mix.dkv": (rank, width), p + "mix.dkv.norm": (rank,), p + "mix.uk": (hd, rank), p + "mix.uv": (hv, rank), p + "mix.sink": (heads,), p + "mix.o": (width, hv)})
+        shapes[p + "mlp.router"] = (n_exp + n_id, width)
+        shapes[p + "mlp.correction"] = (n_exp + n_id,)
+        for e in range(n_exp):
+            shapes[p + "mlp.e%d.up" % e] = (ff, width)
+            shapes[p + "mlp.e%d.down" % e] = (width, ff)
+    os.makedirs(folder, exist_ok=True)
+    head, at = {}, 0
+    for name, shp in shapes.items():
+        n = int(np.prod(shp)) * 2
+        head[name] = {"dtype": "BF16", "shape": list(shp), "data_offsets": [at, at + n]}
+        at += n
+    h = json.dumps(head).encode()
+    h += b" " * (-len(h) % 8)
+    rng = np.random.default_rng(seed)
+    with open(os.path.join(folder, "model.safetensors.part"), "wb") as f:
+        f.write(struct.pack("<Q", len(h)) + h)
+        for name, shp in shapes.items():
+            if len(shp) == 1:
+                v = rng.standard_normal(shp, dtype=np.float32) * 0.1 + (1.0 if name.endswith("mix.norm") or name.endswith("dkv.norm") else 0.0)
+            else:
+                v = rng.standard_normal(shp, dtype=np.float32) * np.float32(shp[-1] ** -0.5)
+            f.write((v.view(np.uint32) >> 16).astype(np.uint16).tobytes())
+    os.replace(os.path.join(folder, "model.safetensors.part"), os.path.join(folder, "model.safetensors"))
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    return folder
+
+
+class KtRow(C.Structure):          # struct pi_kt_row (include/pipeinfer_ops.h)
+    _fields_ = [("family", C.c_int32), ("type", C.c_int32), ("n_tok", C.c_int32), ("sampled_dropped", C.c_int32), ("shape_bytes", C.c_uint64), ("launches", C.c_uint64),
+                ("bytes_total", C.c_double), ("sampled", C.c_uint64), ("avg_us", C.c_double), ("avg_sampled_bytes", C.c_double)]
+
+
+def kernel_table(lib, fn):
+    """runs fn() with every eager launch timed; -> {family: {launches, us, bytes, hbm_frac}}"""
+    lib.pi_kernel_timing(1, 1)
+    fn()
+    L.check(lib.pi_device_sync())
+    buf = (KtRow * 4096)()
+    n = lib.pi_kernel_timing_rows(buf, 4096)
+    lib.pi_kernel_timing(0, 1)
+    out = {}
+    for r in buf[:n]:
+        f = out.setdefault(FAMILIES.get(r.family, "other"), {"launches": 0, "us": 0.0, "bytes": 0.0})
+        f["launches"] += int(r.launches)
+        f["us"] += float(r.avg_us) * int(r.launches)
+        f["bytes"] += float(r.bytes_total)
+    for f in out.values():
+        f["hbm_frac"] = round(f["bytes"] / (f["us"] * 1e-6) / HBM_PEAK, 4) if f["us"] > 0 else None
+        f["us"] = round(f["us"], 1); f["bytes"] = int(f["bytes"])
+    return out
+
+
+def measure(lib, path, n_prompt, n_decode, hybrid, exact=False):
+    model = LL.Model(path)
+    ctx = LL.Context(model, n_ctx=n_prompt + n_decode + 64, n_batch=n_prompt)
+    if hybrid:
+        ctx.set_precision(exact)
+    rng = np.random.default_rng(7)
+    toks = [int(t) for t in rng.integers(1, model.n_vocab, n_prompt + n_decode)]
+    res = {}
+    ctx.feed(toks[:n_prompt], 0, 0)                              # warm-up: upload, graph capture
+    ctx.feed(toks[n_prompt:n_prompt + 2], n_prompt, 0)
+    ctx.seq_rm(0, -1, -1)
+    t_pre = []
+    for _ in range(3):
+        L.check(lib.pi_device_sync()); t0 = time.perf_counter()
+        ctx.feed(toks[:n_prompt], 0, 0)
+        t_pre.append(time.perf_counter() - t0)
+        if _ < 2:
+            ctx.seq_rm(0, -1, -1)
+    t0 = time.perf_counter()
+    for i in range(n_decode):
+        ctx.feed(toks[n_prompt + i:n_prompt + i + 1], n_prompt + i, 0)
+    t_dec = time.perf_counter() - t0
+    res["prefill_tok_s"] = round(n_prompt / sorted(t_pre)[1], 1)
+    res["decode_tok_s"] = round(n_decode / t_dec, 1)
+    res["prefill_ms"] = round(sorted(t_pre)[1] * 1e3, 3)
+    res["decode_ms_per_token"] = round(t_dec / n_decode * 1e3, 4)
+    # kernel by kernel, eager launches (events inside a replayed graph cannot be read): one prompt pass, eight single tokens
+    ctx.seq_rm(0, -1, -1)
+    ctx.set_graphs(False)
+    res["prefill_kernels"] = kernel_table(lib, lambda: ctx.feed(toks[:n_prompt], 0, 0))
+    res["decode_kernels"] = kernel_table(lib, lambda: [ctx.feed(toks[n_prompt + i:n_prompt + i + 1], n_prompt + i, 0) for i in range(8)])
+    ctx.free(); model.free()
+    return res
+
+
+def main(sizes, cache, n_prompt=512, n_decode=64):
+    lib = L.load()
+    L.check(lib.pi_device_init(0), "pi_device_init")
+    from bench import ensure_model
+    for size in sizes:
+        width, n_layer, heads, dim, vdim, rank, n_exp, n_id, top, ff, vocab = SIZES[size]
+        folder = os.path.join(cache, "fasovik-" + size)
+        if not os.path.exists(os.path.join(folder, "model.safetensors")):
+            write_fasovik(folder, size)
+        n_ff = max(32, int(round(2 * top * ff / 3 / 32)) * 32)      # a gated Llama feed-forward with the parameters a token's chosen experts have
+        spec = "cmp-llama-" + size
+        synth.SPECS[spec] = ("llama", n_layer, width, heads, heads, n_ff, vocab, 4096)
+        gguf = ensure_model(cache, spec, "q8_0", 0x5EED, 1.0, 0.25)
+        out = {"size": size, "config": {"width": width, "layers": n_layer, "heads": heads, "dim": dim, "vdim": vdim, "kv_rank": rank, "experts": n_exp, "identity": n_id, "top": top,
+                                       "ff": ff, "vocab": vocab, "n_prompt": n_prompt, "n_decode": n_decode, "llama_n_ff": n_ff},
+               "fasovik_bf16": measure(lib, folder, n_prompt, n_decode, True),
+               "llama_q8_0": measure(lib, gguf, n_prompt, n_decode, False), "data": "synthetic", "hbm_peak": HBM_PEAK}
+        print(json.dumps(out))
+        sys.stdout.flush()
+    return 0

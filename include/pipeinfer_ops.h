@@ -203,6 +203,12 @@ PI_API int pi_op_moe_route(const pi_weight * router, const float * correction_de
 /* out[t] = sum over the chosen outputs e of weight * (e < n_exp ? W_down[e] relu(W_up[e] x[t])^2 : x[t]); w_up: [n_exp * ff][width], w_down: [n_exp * width][ff]; up_dev: scratch [n_tok][top][ff] */
 PI_API int pi_op_moe_experts(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, const float * x_dev, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
                              int exact, float * up_dev, float * out_dev, int64_t out_stride, void * stream);
+/* the same result for a prompt's worth of tokens, serving precision: the (token, choice) slots are sorted by expert on the device and every expert's run goes through the
+ * matrix cores 64 slots at a time.  up_dev: [n_tok * top][ff], dn_dev: [n_tok * top][width], idx_dev: pi_op_moe_grouped_index_ints(n_tok, top, n_exp) int32 */
+PI_API int pi_op_moe_grouped_ok(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, int n_tok, int top, int exact);
+PI_API size_t pi_op_moe_grouped_index_ints(int n_tok, int top, int n_exp);
+PI_API int pi_op_moe_experts_grouped(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, const float * x_dev, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
+                                     float * up_dev, float * dn_dev, int32_t * idx_dev, float * out_dev, int64_t out_stride, void * stream);
 
 #ifdef __cplusplus
 }

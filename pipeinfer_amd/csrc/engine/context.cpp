@@ -40,7 +40,7 @@ llama_context::~llama_context() {
     if (hop_host) (void) hipHostFree(hop_host);
     pi_free(hop_dev);
     pi_free(abort_dev);
-    void * bufs[] = { lat_cache, rec_state, rec_dev, h_in, h_att, h_out, moe_w, moe_up, moe_sel, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
+    void * bufs[] = { lat_cache, rec_state, rec_dev, h_in, h_att, h_out, moe_w, moe_up, moe_dn, moe_sel, moe_idx, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
     for (void * b : bufs) pi_free(b);
     if (rope) pi_rope_table_free(rope);
     if (stream) (void) hipStreamDestroy(stream);
@@ -101,7 +101,7 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
     if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) { err = "hipStreamCreate failed"; return false; }
     auto dev = [&](size_t bytes) -> void * { void * p = pi_malloc(std::max<size_t>(bytes, 16)); if (!p) err = pi_last_error(); return p; };
     const int nb = ctx->n_batch, width = hp.n_embd;
-    size_t lat = 0, rec = 0, in_w = 1, att_w = 1, up_w = 1, sel_w = 1;
+    size_t lat = 0, rec = 0, in_w = 1, att_w = 1, up_w = 1, sel_w = 1, idx_n = 1;
     ctx->lat_off.assign(hp.hybrid.size(), 0); ctx->rec_off.assign(hp.hybrid.size(), 0);
     if (hp.n_recurrent() > 0) ctx->slots.reset(new state_slots(std::max(1, ctx->n_state_slots)));
     for (size_t i = 0; i < hp.hybrid.size(); i++) {
@@ -112,13 +112,13 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
         }
         if (H.state_index >= 0) { ctx->rec_off[i] = rec; rec += (size_t) ctx->slots->size() * H.heads * H.dim * H.vdim; }
         in_w = std::max(in_w, (size_t) H.in_rows()); att_w = std::max(att_w, (size_t) H.heads * H.vdim);
-        if (H.has_mlp) { up_w = std::max(up_w, (size_t) H.top * std::max(H.ff, 1)); sel_w = std::max(sel_w, (size_t) H.top); }
+        if (H.has_mlp) { up_w = std::max(up_w, (size_t) H.top * std::max(H.ff, 1)); sel_w = std::max(sel_w, (size_t) H.top); idx_n = std::max(idx_n, pi_op_moe_grouped_index_ints(nb, H.top, H.n_expert)); }
     }
     if (!(ctx->lat_cache = (float *) dev(lat * 4)) || !(ctx->rec_state = (float *) dev(rec * 4))) return false;
     pi_memset(ctx->lat_cache, 0, std::max<size_t>(lat * 4, 16), nullptr); pi_memset(ctx->rec_state, 0, std::max<size_t>(rec * 4, 16), nullptr);
     if (!(ctx->x = (float *) dev((size_t) 4 * nb * width)) || !(ctx->nx = (float *) dev((size_t) 4 * nb * width)) || !(ctx->h_out = (float *) dev((size_t) 4 * nb * width)) ||
         !(ctx->h_in = (float *) dev((size_t) 4 * nb * in_w)) || !(ctx->h_att = (float *) dev((size_t) 4 * nb * att_w)) || !(ctx->moe_up = (float *) dev((size_t) 4 * nb * up_w)) ||
-        !(ctx->moe_w = (float *) dev((size_t) 4 * nb * sel_w)) || !(ctx->moe_sel = (int32_t *) dev((size_t) 4 * nb * sel_w)) || (ctx->slots && !(ctx->rec_dev = (int32_t *) dev((size_t) 4 * nb))) ||
+        !(ctx->moe_w = (float *) dev((size_t) 4 * nb * sel_w)) || !(ctx->moe_dn = (float *) dev((size_t) 4 * nb * sel_w * width)) || !(ctx->moe_idx = (int32_t *) dev((size_t) 4 * idx_n)) || !(ctx->moe_sel = (int32_t *) dev((size_t) 4 * nb * sel_w)) || (ctx->slots && !(ctx->rec_dev = (int32_t *) dev((size_t) 4 * nb))) ||
         !(ctx->tokens_dev = (int32_t *) dev((size_t) 4 * nb)) || !(ctx->pos_dev = (int32_t *) dev((size_t) 4 * nb)) || !(ctx->dyn_dev = (int32_t *) dev((size_t) 4 * (4 + 2 * nb))))
         return false;
     {   // abort word + cancel flags + the control stream cancels travel on
@@ -303,7 +303,10 @@ static bool forward_hybrid(llama_context * ctx, int n_tok, int n_kv) {
         OP_OK(pi_op_rms_scale(Y, width, W.norm1, 1.0f, eps, width, n_tok, nullptr, 0, x, width, rm, x, width, nullptr, 0, s));
         if (H.has_mlp) {
             OP_OK(pi_op_moe_route(W.router, W.correction, x, width, n_tok, H.top, ex, ctx->moe_sel, ctx->moe_w, s));
-            OP_OK(pi_op_moe_experts(W.e_up, W.e_down, H.n_expert, H.ff, x, width, ctx->moe_sel, ctx->moe_w, n_tok, H.top, ex, ctx->moe_up, Y, width, s));
+            if (pi_op_moe_grouped_ok(W.e_up, W.e_down, H.n_expert, H.ff, n_tok, H.top, ex))                                                        // prompts: by expert, on the matrix cores
+                OP_OK(pi_op_moe_experts_grouped(W.e_up, W.e_down, H.n_expert, H.ff, x, width, ctx->moe_sel, ctx->moe_w, n_tok, H.top, ctx->moe_up, ctx->moe_dn, ctx->moe_idx, Y, width, s));
+            else
+                OP_OK(pi_op_moe_experts(W.e_up, W.e_down, H.n_expert, H.ff, x, width, ctx->moe_sel, ctx->moe_w, n_tok, H.top, ex, ctx->moe_up, Y, width, s));
             OP_OK(pi_op_rms_scale(Y, width, W.norm2, 1.0f, eps, width, n_tok, nullptr, 0, x, width, rm, x, width, nullptr, 0, s));
         }
         trace(ctx, "lout", (int) il, x, width, n_tok);

@@ -407,3 +407,134 @@ extern "C" int pi_op_moe_experts(const pi_weight * wup, const pi_weight * wdown,
                  n_exp > 0 ? (const uint16_t *) wdown->p0 : nullptr, width, ff, n_exp, top, x, x_stride, sel_dev, selw_dev, up_dev, exact, out, out_stride, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
 }
+
+// ---- the same for a prompt's worth of tokens: grouped by expert, on the matrix cores ---------------------------------------------------------------------
+// k_moe_group sorts the (token, choice) slots of a pass by expert (a counting sort in one workgroup) and cuts every expert's run into tiles of 64 slots; k_moe_up_mfma /
+// k_moe_down_mfma compute 64 slots x 64 rows per workgroup with v_mfma_f32_16x16x32_bf16 (operand layout as k_dense_mfma: A = 16 weight rows, B = 16 slots, 8 consecutive k per
+// lane) — an expert's matrices are read once per 64 of its tokens instead of once per token; k_moe_combine sums a token's weighted choices (identity experts: the input itself).
+// idx layout (int32): [0] number of tiles | tile expert [max_tiles] | tile start [max_tiles] | tile length [max_tiles] | order [n_slots]
+typedef __bf16 hy_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float hy_f32x4 __attribute__((ext_vector_type(4)));
+typedef uint16_t hy_u16x8 __attribute__((ext_vector_type(8)));
+#define MOE_GROUP_MAX_EXPERTS 1024
+static inline int moe_max_tiles(int n_slots, int n_exp) { return (n_slots + 63) / 64 + std::min(n_exp, n_slots); }
+
+__global__ void __launch_bounds__(256) k_moe_group(const int32_t * __restrict__ sel, int n_slots, int n_exp, int max_tiles, int32_t * __restrict__ idx, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    __shared__ int cnt[MOE_GROUP_MAX_EXPERTS], cur[MOE_GROUP_MAX_EXPERTS];
+    int32_t * tile_e = idx + 1, * tile_s = tile_e + max_tiles, * tile_n = tile_s + max_tiles, * order = tile_n + max_tiles;
+    for (int e = threadIdx.x; e < n_exp; e += 256) cnt[e] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n_slots; i += 256) { const int e = sel[i]; if (e >= 0 && e < n_exp) atomicAdd(&cnt[e], 1); }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0, nt = 0;
+        for (int e = 0; e < n_exp; e++) {
+            cur[e] = at;
+            for (int k = 0; k < cnt[e]; k += 64) { tile_e[nt] = e; tile_s[nt] = at + k; tile_n[nt] = min(64, cnt[e] - k); nt++; }
+            at += cnt[e];
+        }
+        idx[0] = nt;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n_slots; i += 256) { const int e = sel[i]; if (e >= 0 && e < n_exp) order[atomicAdd(&cur[e], 1)] = i; }
+}
+
+// acc[j] += W[rows j*16 + (l % 16)][k] * B[slot (l % 16)][k] over K (K % 8 == 0); brow: this lane's B row (nullptr: zeros), wrow[j]: this lane's A rows (nullptr: zeros)
+static __device__ __forceinline__ void hy_mfma_rows(const uint16_t * const wrow[4], const float * brow, int64_t K, int kb, hy_f32x4 acc[4]) {
+    for (int64_t k0 = 0; k0 < K; k0 += 32) {
+        const int64_t k = k0 + kb * 8;
+        const bool k_ok = k < K;
+        hy_u16x8 b = hy_u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (k_ok && brow) {
+            const float4 v0 = *(const float4 *) (brow + k), v1 = *(const float4 *) (brow + k + 4);
+            const float f[8] = { v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w };
+#pragma unroll
+            for (int i = 0; i < 8; i++) { const uint32_t u = __float_as_uint(f[i]); b[i] = (uint16_t) ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16); }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            hy_u16x8 a = hy_u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (k_ok && wrow[j]) a = *(const hy_u16x8 *) (wrow[j] + k);
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(hy_bf16x8, a), __builtin_bit_cast(hy_bf16x8, b), acc[j], 0, 0, 0);
+        }
+    }
+}
+
+// UP: B rows are the tokens' inputs x[slot / top], A rows W_up[e], out up[slot][f] = relu(.)^2;  !UP: B rows up[slot] (K = ff), A rows W_down[e], out dn[slot][n]
+template <bool UP>
+__global__ void __launch_bounds__(256) k_moe_mfma(const uint16_t * __restrict__ W, int64_t K, int rows, const float * __restrict__ B, int64_t bs, int top, const int32_t * __restrict__ idx,
+                                                  int max_tiles, float * __restrict__ out, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w, 1)) return;
+    const int tile = blockIdx.y;
+    if (tile >= idx[0]) return;
+    const int32_t * tile_e = idx + 1, * tile_s = tile_e + max_tiles, * tile_n = tile_s + max_tiles, * order = tile_n + max_tiles;
+    const int e = tile_e[tile], start = tile_s[tile], len = tile_n[tile];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, kb = lane >> 4;
+    if (wave * 16 >= len) return;                                  // (whole waves: no barrier follows)
+    const int si = wave * 16 + li;
+    const int slot = si < len ? order[start + si] : -1;
+    const float * brow = slot < 0 ? nullptr : B + (int64_t) (UP ? slot / top : slot) * bs;
+    const int n0 = blockIdx.x * 64;
+    const uint16_t * wrow[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) { const int r = n0 + j * 16 + li; wrow[j] = r < rows ? W + ((int64_t) e * rows + r) * K : nullptr; }
+    hy_f32x4 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[j] = hy_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    hy_mfma_rows(wrow, brow, K, kb, acc);
+    if (slot < 0) return;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int row = n0 + j * 16 + kb * 4 + r;
+            if (row < rows) { float v = acc[j][r]; if (UP) { v = fmaxf(v, 0.0f); v *= v; } out[(int64_t) slot * rows + row] = v; }
+        }
+}
+
+__global__ void __launch_bounds__(256) k_moe_combine(const float * __restrict__ dn, int64_t width, int n_exp, int top, const float * __restrict__ x, int64_t xs, const int32_t * __restrict__ sel,
+                                                     const float * __restrict__ selw, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.y;
+    const int64_t n = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (n >= width) return;
+    float acc = 0.0f;
+    for (int kk = 0; kk < top; kk++) {
+        const int e = sel[(int64_t) t * top + kk];
+        acc = fmaf(selw[(int64_t) t * top + kk], e >= n_exp ? x[(int64_t) t * xs + n] : dn[((int64_t) t * top + kk) * width + n], acc);
+    }
+    out[(int64_t) t * os + n] = acc;
+}
+
+// ints of index scratch the grouped path needs for a pass of n_tok tokens
+extern "C" size_t pi_op_moe_grouped_index_ints(int n_tok, int top, int n_exp) { const int ns = n_tok * top; return (size_t) 1 + 3 * (size_t) moe_max_tiles(ns, n_exp) + (size_t) ns; }
+// whether a pass of this shape takes the grouped matrix-core path (otherwise pi_op_moe_experts: gathered mat-vecs)
+extern "C" int pi_op_moe_grouped_ok(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, int n_tok, int top, int exact) {
+    static const int min_slots = getenv("PI_MOE_GROUPED_MIN") ? atoi(getenv("PI_MOE_GROUPED_MIN")) : 32;
+    return !exact && n_exp > 0 && n_exp <= MOE_GROUP_MAX_EXPERTS && wup && wdown && n_tok * top >= min_slots && wup->ne0 % 8 == 0 && ff % 8 == 0 &&
+           ((uintptr_t) wup->p0 % 16) == 0 && ((uintptr_t) wdown->p0 % 16) == 0;
+}
+// up_dev: [n_tok * top][ff], dn_dev: [n_tok * top][width], idx_dev: pi_op_moe_grouped_index_ints ints
+extern "C" int pi_op_moe_experts_grouped(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, const float * x, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
+                                         float * up_dev, float * dn_dev, int32_t * idx_dev, float * out, int64_t out_stride, void * stream) {
+    if (!pi_op_moe_grouped_ok(wup, wdown, n_exp, ff, n_tok, top, 0)) { pi_set_error("pi_op_moe_experts_grouped: this shape takes pi_op_moe_experts"); return -1; }
+    if (wup->type != PI_BF16 || wdown->type != PI_BF16 || wup->ne1 != (int64_t) n_exp * ff || wdown->ne0 != ff || wdown->ne1 != (int64_t) n_exp * wup->ne0 || x_stride % 4 || ((uintptr_t) x % 16)) {
+        pi_set_error("pi_op_moe_experts_grouped: expert matrices must be bfloat16 [experts * ff][width] and [experts * width][ff], inputs 16-byte aligned rows"); return -1;
+    }
+    hipStream_t s = (hipStream_t) stream;
+    const int64_t width = wup->ne0;
+    const int ns = n_tok * top, mt = moe_max_tiles(ns, n_exp), nta = std::min(n_tok, PI_KT_MAXNT - 1);
+    const double wbytes = std::min<double>(ns, n_exp) * 2.0 * ff * width;
+    PI_KT_LAUNCH(PI_KT_OTHER, PI_BF16, 1, 8.0 * ns, k_moe_group, dim3(1), dim3(256), 0, s, sel_dev, ns, n_exp, mt, idx_dev, pi_abort_word());
+    PI_CHECK_LAUNCH();
+    PI_KT_LAUNCH(PI_KT_MMQ, PI_BF16, nta, wbytes + 4.0 * ns * (width + ff), k_moe_mfma<true>, dim3((unsigned) ((ff + 63) / 64), (unsigned) mt), dim3(256), 0, s,
+                 (const uint16_t *) wup->p0, width, ff, x, x_stride, top, idx_dev, mt, up_dev, pi_abort_word());
+    PI_CHECK_LAUNCH();
+    PI_KT_LAUNCH(PI_KT_MMQ, PI_BF16, nta, wbytes + 4.0 * ns * (width + ff), k_moe_mfma<false>, dim3((unsigned) ((width + 63) / 64), (unsigned) mt), dim3(256), 0, s,
+                 (const uint16_t *) wdown->p0, (int64_t) ff, (int) width, up_dev, (int64_t) ff, top, idx_dev, mt, dn_dev, pi_abort_word());
+    PI_CHECK_LAUNCH();
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 4.0 * n_tok * width * (top + 2), k_moe_combine, dim3((unsigned) ((width + 255) / 256), (unsigned) n_tok), dim3(256), 0, s,
+                 dn_dev, width, n_exp, top, x, x_stride, sel_dev, selw_dev, out, out_stride, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}

@@ -390,7 +390,7 @@ def test_three_processes_on_one_gpu_through_the_library_transport(tmp_path, tgt,
     for s in v["stages"]:
         hop_gpu_us, hop_host_us = 1e3 * s["hop_gpu_ms"] / s["runs"], 1e3 * s["send_ms"] / s["received"]
         print(f"stage {s['rank']}: store of the activations / logits {hop_gpu_us:.1f} us of GPU time per run, header published {hop_host_us:.1f} us after the run; waited {s['wait_out_ms']:.2f} ms in all for a free slot downstream")
-        if not host_rings:
+        if not host_rings and s["device_flags"]:                                                 # (host-published headers — a box that cannot map the control block — are the host-mediated hop itself)
             assert hop_gpu_us < 50.0 and hop_host_us < 50.0, s
     # device-side arrival flags (the default in device mode): every run is announced downstream before it is computed and the consuming stage's run is enqueued behind a
     # device-side wait; the flag written by the producing stage's STREAM (behind its peer store) is seen by the waiting kernel within microseconds — no host thread on the

@@ -192,11 +192,14 @@ PI_API int pi_op_linear_attention(const float * q_dev, const float * k_dev, cons
                                   const int32_t * rec_dev, int n_tok, int max_segments, float * out_dev, int64_t out_stride, void * stream);
 PI_API int pi_op_copy_f32(const float * src_dev, float * dst_dev, int64_t n, void * stream);
 /* Attention over a cache of latents c [cells][rank] fp32 shared by all heads: k = W_uk c, v = W_uv c per head, never materialised (W_uk is folded into the query, W_uv applied to
- * the weighted sum of latents); score = q . k * scale; soft-max whose denominator also holds exp(sink[h]).  mask_dev / n_kv / dyn_dev as for pi_op_attention_ex (single run). */
+ * the weighted sum of latents); score = q . k * scale; soft-max whose denominator also holds exp(sink[h]).  mask_dev / n_kv / dyn_dev as for pi_op_attention_ex (single run).
+ * scratch_dev: pi_op_latent_attention_scratch_floats(heads, rank, widest pass, n_kv) floats (folded queries and the partial results of the cell-range splits) */
 PI_API int pi_op_latent_attention(const float * q_dev, int64_t q_stride, const float * cache_dev, const uint32_t * mask_dev, const pi_weight * w_uk, const pi_weight * w_uv, const float * sink_dev,
-                                  float scale, int heads, int dim, int vdim, int rank, int n_tok, int n_kv, float * out_dev, int64_t out_stride, const int32_t * dyn_dev, void * stream);
-PI_API int pi_op_latent_attention_reserve(void);                   /* once per process, outside graph capture: LDS limit for long contexts */
-PI_API int pi_op_latent_attention_max_cells(int rank);             /* longest context the kernel serves at this latent width */
+                                  float scale, int heads, int dim, int vdim, int rank, int n_tok, int n_kv, float * scratch_dev, size_t scratch_floats, float * out_dev, int64_t out_stride,
+                                  const int32_t * dyn_dev, void * stream);
+PI_API size_t pi_op_latent_attention_scratch_floats(int heads, int rank, int n_tok, int n_kv);
+PI_API int pi_op_latent_attention_reserve(void);                   /* once per process, outside graph capture: LDS limit of the score kernels */
+PI_API int pi_op_latent_attention_max_cells(int rank);             /* longest context the kernels serve */
 /* Router of a mixture of experts: scores = softmax(W_router x) over all outputs; the `top` outputs with the largest score + correction are chosen (lowest index wins a tie); their
  * weights are the scores themselves.  sel_dev / selw_dev: [n_tok][top] */
 PI_API int pi_op_moe_route(const pi_weight * router, const float * correction_dev, const float * x_dev, int64_t x_stride, int n_tok, int top, int exact, int32_t * sel_dev, float * selw_dev, void * stream);

@@ -40,7 +40,7 @@ llama_context::~llama_context() {
     if (hop_host) (void) hipHostFree(hop_host);
     pi_free(hop_dev);
     pi_free(abort_dev);
-    void * bufs[] = { lat_cache, rec_state, rec_dev, h_in, h_att, h_out, moe_w, moe_up, moe_dn, moe_sel, moe_idx, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
+    void * bufs[] = { lat_cache, rec_state, rec_dev, h_in, h_att, h_out, moe_w, moe_up, moe_dn, lat_scratch, moe_sel, moe_idx, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
     for (void * b : bufs) pi_free(b);
     if (rope) pi_rope_table_free(rope);
     if (stream) (void) hipStreamDestroy(stream);
@@ -109,12 +109,13 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
         if (H.cache_index >= 0) {
             if (ctx->n_ctx > pi_op_latent_attention_max_cells(H.kv_rank)) { err = "n_ctx = " + std::to_string(ctx->n_ctx) + " is beyond the latent-attention kernel at kv_rank " + std::to_string(H.kv_rank) + " (one score row per workgroup in LDS: n_ctx <= " + std::to_string(pi_op_latent_attention_max_cells(H.kv_rank)) + ")"; return false; }
             ctx->lat_off[i] = lat; lat += (size_t) ctx->n_ctx * H.kv_rank;
+            ctx->lat_scratch_floats = std::max(ctx->lat_scratch_floats, pi_op_latent_attention_scratch_floats(H.heads, H.kv_rank, nb, ctx->n_ctx));
         }
         if (H.state_index >= 0) { ctx->rec_off[i] = rec; rec += (size_t) ctx->slots->size() * H.heads * H.dim * H.vdim; }
         in_w = std::max(in_w, (size_t) H.in_rows()); att_w = std::max(att_w, (size_t) H.heads * H.vdim);
         if (H.has_mlp) { up_w = std::max(up_w, (size_t) H.top * std::max(H.ff, 1)); sel_w = std::max(sel_w, (size_t) H.top); idx_n = std::max(idx_n, pi_op_moe_grouped_index_ints(nb, H.top, H.n_expert)); }
     }
-    if (!(ctx->lat_cache = (float *) dev(lat * 4)) || !(ctx->rec_state = (float *) dev(rec * 4))) return false;
+    if (!(ctx->lat_scratch = (float *) dev(ctx->lat_scratch_floats * 4)) || !(ctx->lat_cache = (float *) dev(lat * 4)) || !(ctx->rec_state = (float *) dev(rec * 4))) return false;
     pi_memset(ctx->lat_cache, 0, std::max<size_t>(lat * 4, 16), nullptr); pi_memset(ctx->rec_state, 0, std::max<size_t>(rec * 4, 16), nullptr);
     if (!(ctx->x = (float *) dev((size_t) 4 * nb * width)) || !(ctx->nx = (float *) dev((size_t) 4 * nb * width)) || !(ctx->h_out = (float *) dev((size_t) 4 * nb * width)) ||
         !(ctx->h_in = (float *) dev((size_t) 4 * nb * in_w)) || !(ctx->h_att = (float *) dev((size_t) 4 * nb * att_w)) || !(ctx->moe_up = (float *) dev((size_t) 4 * nb * up_w)) ||
@@ -291,7 +292,7 @@ static bool forward_hybrid(llama_context * ctx, int n_tok, int n_kv) {
             float * cache = ctx->lat_cache + ctx->lat_off[il];
             OP_OK(pi_op_dense(W.w_in, x, width, n_tok, P, pw, PI_ACT_NONE, pw, PI_ACT_NONE, ex, s));                                               // q | W_dkv h
             OP_OK(pi_op_rms_scale(P + hd, pw, W.mix_norm, 0.0f, eps, H.kv_rank, n_tok, nullptr, 0, nullptr, 0, 1.0f, cache, H.kv_rank, ctx->dyn_dev, 1, s));   // the latent, into its cell
-            OP_OK(pi_op_latent_attention(P, pw, cache, ctx->mask_dev, W.w_uk, W.w_uv, W.sink, H.scale, H.heads, H.dim, H.vdim, H.kv_rank, n_tok, n_kv, A, hv, ctx->dyn_dev, s));
+            OP_OK(pi_op_latent_attention(P, pw, cache, ctx->mask_dev, W.w_uk, W.w_uv, W.sink, H.scale, H.heads, H.dim, H.vdim, H.kv_rank, n_tok, n_kv, ctx->lat_scratch, ctx->lat_scratch_floats, A, hv, ctx->dyn_dev, s));
         } else {
             float * state = ctx->rec_state + ctx->rec_off[il];
             OP_OK(pi_op_dense(W.w_in, x, width, n_tok, P, pw, PI_ACT_SILU, 2 * hd + hv, PI_ACT_SIGMOID, ex, s));                                   // silu(q | k | v) | sigmoid(g)

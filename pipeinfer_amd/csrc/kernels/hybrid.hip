@@ -16,6 +16,25 @@
 static __device__ __forceinline__ float hy_widen(uint16_t b) { return __uint_as_float((uint32_t) b << 16); }
 static __device__ __forceinline__ float hy_round(float f) { const uint32_t u = __float_as_uint(f); return __uint_as_float(((u + 0x7fffu + ((u >> 16) & 1u)) >> 16) << 16); }
 
+typedef uint16_t hy_u16x8v __attribute__((ext_vector_type(8)));
+// this lane's share of w . x over n values (bfloat16 row w, fp32 row x); vec: n % 8 == 0 and both rows 16-byte aligned — 16-byte weight loads, several in flight
+static __device__ __forceinline__ float hy_dot_lane(const uint16_t * __restrict__ w, const float * __restrict__ x, int64_t n, int lane, bool exact, bool vec) {
+    float a = 0.0f;
+    if (vec) {
+#pragma unroll 4
+        for (int64_t i = (int64_t) lane * 8; i < n; i += 512) {
+            const hy_u16x8v wv = *(const hy_u16x8v *) (w + i);
+            const float4 x0 = *(const float4 *) (x + i), x1 = *(const float4 *) (x + i + 4);
+            const float xf[8] = { x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w };
+#pragma unroll
+            for (int k = 0; k < 8; k++) a = fmaf(hy_widen(wv[k]), exact ? xf[k] : hy_round(xf[k]), a);
+        }
+    } else {
+        for (int64_t i = lane; i < n; i += 64) a = fmaf(hy_widen(w[i]), exact ? x[i] : hy_round(x[i]), a);
+    }
+    return a;
+}
+
 // sum over the 256 threads of a block (every thread gets the total); red: 4 floats of LDS, reusable after the call
 static __device__ __forceinline__ float hy_block_sum(float v, float * red) {
     v = pi_lanes_sum<64>(v);
@@ -39,16 +58,29 @@ static __device__ __forceinline__ float hy_block_max(float v, float * red) {
 // ---- RMS norm with its usual companions ---------------------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256) k_rms_scale(const float * __restrict__ x, int64_t xs, const float * __restrict__ w, float w_off, float eps, int n,
                                                    const float * __restrict__ gate, int64_t gs, const float * __restrict__ res, int64_t rs, float mult,
-                                                   float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn, int to_cells, const int32_t * __restrict__ abort_w) {
+                                                   float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn, int to_cells, int vec, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     __shared__ float red[4];
     const int t = blockIdx.x;
     const float * xr = x + (int64_t) t * xs;
     float ss = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
+    if (vec) { for (int i = threadIdx.x * 4; i < n; i += 1024) { const float4 v = *(const float4 *) (xr + i); ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss); } }
+    else for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
     ss = hy_block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float) n + eps);
     const int64_t orow = to_cells ? pi_cell_of(dyn, 0, t) : t;
+    if (vec) {
+        for (int i = threadIdx.x * 4; i < n; i += 1024) {
+            const float4 xv = *(const float4 *) (xr + i), wv = *(const float4 *) (w + i);
+            float y[4] = { xv.x * inv * (wv.x + w_off), xv.y * inv * (wv.y + w_off), xv.z * inv * (wv.z + w_off), xv.w * inv * (wv.w + w_off) };
+            if (gate) { const float4 g = *(const float4 *) (gate + (int64_t) t * gs + i); y[0] *= g.x; y[1] *= g.y; y[2] *= g.z; y[3] *= g.w; }
+#pragma unroll
+            for (int k = 0; k < 4; k++) y[k] *= mult;
+            if (res) { const float4 r = *(const float4 *) (res + (int64_t) t * rs + i); y[0] = r.x + y[0]; y[1] = r.y + y[1]; y[2] = r.z + y[2]; y[3] = r.w + y[3]; }
+            *(float4 *) (out + orow * os + i) = make_float4(y[0], y[1], y[2], y[3]);
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < n; i += 256) {
         float y = xr[i] * inv * (w[i] + w_off);
         if (gate) y *= gate[(int64_t) t * gs + i];
@@ -62,25 +94,27 @@ extern "C" int pi_op_rms_scale(const float * x, int64_t x_stride, const float * 
                                const float * residual, int64_t residual_stride, float mult, float * out, int64_t out_stride, const int32_t * dyn_dev, int to_cells, void * stream) {
     if (n_tok <= 0 || n <= 0) return 0;
     if (to_cells && !dyn_dev) { pi_set_error("pi_op_rms_scale: rows go to cache cells but no cell table was given"); return -1; }
+    auto al = [](const void * p, int64_t stride) { return !p || (((uintptr_t) p % 16) == 0 && stride % 4 == 0); };
+    const int vec = n % 4 == 0 && al(x, x_stride) && al(w, 0) && al(gate, gate_stride) && al(residual, residual_stride) && al(out, out_stride);
     PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 12.0 * n * n_tok, k_rms_scale, dim3((unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, x, x_stride, w, w_offset, eps, n, gate, gate_stride,
-                 residual, residual_stride, mult, out, out_stride, dyn_dev, to_cells, pi_abort_word());
+                 residual, residual_stride, mult, out, out_stride, dyn_dev, to_cells, vec, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
 }
 
 // ---- linear attention with a per-head decay -------------------------------------------------------------------------------------------------------
 // rec[t] = state slot of token t (| 1 << 30 on the first token of a sequence whose state starts from zero), tokens of one slot are consecutive.  Workgroup (head, column block,
 // segment ordinal): thread (column j, part sp of R) keeps S[i][j] for its DPT rows i in registers, walks the segment's tokens in order and leaves S in HBM.
-#define LA_TB 16                                  // tokens whose q and k are staged in LDS at a time
+#define LA_TB 32                                  // tokens whose q, k and v are staged in LDS at a time
 #define LA_FRESH (1 << 30)
 template <int DPT>
 __global__ void __launch_bounds__(256) k_linear_attention(const float * __restrict__ q, const float * __restrict__ k, const float * __restrict__ v, int64_t stride, int heads, int dim, int vdim, int R,
                                                           const float * __restrict__ decay, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
                                                           float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
-    extern __shared__ float lds[];                // q tile [LA_TB][dim] | k tile [LA_TB][dim] | the slot words of the pass [n_tok]
+    extern __shared__ float lds[];                // q tile [LA_TB][dim] | k tile [LA_TB][dim] | v tile [LA_TB][cols] | the slot words of the pass [n_tok]
     __shared__ int seg[3];                        // first token, length, slot word
     const int h = blockIdx.x, tid = threadIdx.x;
-    int * recs = (int *) (lds + 2 * LA_TB * dim);
+    int * recs = (int *) (lds + 2 * LA_TB * dim + LA_TB * (blockDim.x / R));
     for (int t = tid; t < n_tok; t += blockDim.x) recs[t] = rec[t];
     __syncthreads();
     if (tid == 0) {
@@ -108,7 +142,8 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
         const int i = sp * DPT + ii;
         S[ii] = (col_ok && i < dim && !(word & LA_FRESH)) ? S_hbm[(int64_t) i * vdim + j] : 0.0f;
     }
-    float * qt = lds, * kt = lds + LA_TB * dim;
+    float * qt = lds, * kt = lds + LA_TB * dim, * vt = kt + LA_TB * dim;
+    const bool dim4 = (dim & 3) == 0;
     for (int t0 = 0; t0 < len; t0 += LA_TB) {
         const int nt = min(LA_TB, len - t0);
         __syncthreads();
@@ -117,21 +152,33 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
             const int64_t off = (int64_t) (first + t0 + tt) * stride + (int64_t) h * dim + i;
             qt[idx] = q[off]; kt[idx] = k[off];
         }
+        for (int idx = tid; idx < nt * cols; idx += blockDim.x) {
+            const int tt = idx / cols, jj = blockIdx.y * cols + idx % cols;
+            vt[idx] = jj < vdim ? v[(int64_t) (first + t0 + tt) * stride + (int64_t) h * vdim + jj] : 0.0f;
+        }
         __syncthreads();
         for (int tt = 0; tt < nt; tt++) {
-            const int t = first + t0 + tt;
-            const float vj = col_ok ? v[(int64_t) t * stride + (int64_t) h * vdim + j] : 0.0f;
+            const float vj = vt[tt * cols + tid / R];
+            const float * kr = kt + tt * dim + sp * DPT, * qr = qt + tt * dim + sp * DPT;
             float o = 0.0f;
+            if (dim4) {
 #pragma unroll
-            for (int ii = 0; ii < DPT; ii++) {
-                const int i = sp * DPT + ii;
-                if (i < dim) {
-                    S[ii] = fmaf(kt[tt * dim + i], vj, lam * S[ii]);
-                    o = fmaf(S[ii], qt[tt * dim + i], o);
+                for (int ii = 0; ii < DPT; ii += 4) {
+                    if (sp * DPT + ii < dim) {
+                        const float4 kv = *(const float4 *) (kr + ii), qv = *(const float4 *) (qr + ii);
+                        S[ii] = fmaf(kv.x, vj, lam * S[ii]);         o = fmaf(S[ii], qv.x, o);
+                        S[ii + 1] = fmaf(kv.y, vj, lam * S[ii + 1]); o = fmaf(S[ii + 1], qv.y, o);
+                        S[ii + 2] = fmaf(kv.z, vj, lam * S[ii + 2]); o = fmaf(S[ii + 2], qv.z, o);
+                        S[ii + 3] = fmaf(kv.w, vj, lam * S[ii + 3]); o = fmaf(S[ii + 3], qv.w, o);
+                    }
                 }
+            } else {
+#pragma unroll
+                for (int ii = 0; ii < DPT; ii++)
+                    if (sp * DPT + ii < dim) { S[ii] = fmaf(kr[ii], vj, lam * S[ii]); o = fmaf(S[ii], qr[ii], o); }
             }
             for (int d = R >> 1; d > 0; d >>= 1) o += __shfl_xor(o, d, PI_WAVE);
-            if (col_ok && sp == 0) out[(int64_t) t * os + (int64_t) h * vdim + j] = o;
+            if (col_ok && sp == 0) out[(int64_t) (first + t0 + tt) * os + (int64_t) h * vdim + j] = o;
         }
     }
     if (col_ok)
@@ -148,7 +195,7 @@ extern "C" int pi_op_linear_attention(const float * q, const float * k, const fl
     int threads = std::min(256, (vdim * R + 63) / 64 * 64);
     const int cols = threads / R;
     const dim3 grid((unsigned) heads, (unsigned) ((vdim + cols - 1) / cols), (unsigned) std::max(1, std::min(n_tok, max_segments)));
-    const size_t lds = ((size_t) 2 * LA_TB * dim + (size_t) n_tok) * sizeof(float);
+    const size_t lds = ((size_t) 2 * LA_TB * dim + (size_t) LA_TB * cols + (size_t) n_tok) * sizeof(float);
     const double bytes = 4.0 * n_tok * heads * (2.0 * dim + 2.0 * vdim) + 8.0 * heads * dim * vdim;
     hipStream_t s = (hipStream_t) stream;
 #define LA_GO(D) PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), bytes, k_linear_attention<D>, grid, dim3(threads), lds, s, q, k, v, stride, heads, dim, vdim, R, decay_dev, state_dev, rec_dev, n_tok, out, out_stride, pi_abort_word())
@@ -168,155 +215,343 @@ extern "C" int pi_op_copy_f32(const float * src, float * dst, int64_t n, void * 
 }
 
 // ---- attention over a shared latent -----------------------------------------------------------------------------------------------------------------
-// grid (token, head tile of HT); LDS: qa [HT][rank] (absorbed, pre-scaled queries) | ol [4 waves][HT][rank] | sc [HT][cap] scores then probabilities
-template <int HT>
-__global__ void __launch_bounds__(256) k_latent_attention(const float * __restrict__ q, int64_t qs, const float * __restrict__ cache, const uint32_t * __restrict__ mask,
-                                                          const uint16_t * __restrict__ wuk, const uint16_t * __restrict__ wuv, const float * __restrict__ sink, float scale,
-                                                          int heads, int dim, int vdim, int rank, int n_kv_arg, int cap, float * __restrict__ out, int64_t os,
-                                                          const int32_t * __restrict__ dyn, const int32_t * __restrict__ abort_w) {
+// Three launches.  (1) k_latent_absorb folds the key up-projection and the score scale into the query: qa[t][h][:] = scale * W_uk[h]^T q[t][h] (rank values per head).
+// (2) k_latent_scores, grid (token, head tile of M heads, split of the cell range): a thread owns a cell in the score phase — its latent row streams through registers once and
+// feeds M accumulators, the M queries come through wave-uniform (scalar) loads — and a slice of the latent's rank in the value phase, where the probabilities of a cell are
+// broadcast from LDS to M x RPT accumulators; every split leaves an un-normalised partial (max, sum, sum of p * c) in scratch.  (3) k_latent_combine merges the splits with
+// the sink term, normalises and applies the value up-projection.  K / V are never materialised; single tokens are spread over the chip by the splits (64 cells each),
+// prompts take splits only when a score row would not fit LDS.
+// scratch (floats): qa [n_tok][heads][rank] | pol [n_tok][heads][S][rank] | pml [n_tok][heads][S][2]
+#define LAT_LDS_BUDGET (128 * 1024)
+struct lat_plan { int M, RPT, cap, S; size_t lds, scratch; };
+static lat_plan latent_plan(int heads, int rank, int n_tok, int n_ctx) {
+    lat_plan p;
+    const bool single = n_tok <= 8;
+    int best = 1;                                                     // heads per workgroup: the largest tile that leaves at most a quarter of its accumulator rows idle
+    for (int m : { 2, 4, 8, 16 }) { if (single && m > 4) break; if (3 * ((heads + m - 1) / m * m) <= 4 * heads) best = m; }
+    p.M = best;
+    p.RPT = rank > 512 ? 4 : rank > 256 ? 2 : 1;
+    const int rthreads = (rank + p.RPT - 1) / p.RPT, G = std::max(1, 256 / rthreads);
+    const int cap_max = std::max(64, (int) (((LAT_LDS_BUDGET / 4 - (size_t) G * p.M * rank - 256 * p.M) / p.M) / 64 * 64));
+    p.cap = single ? 64 : std::min(cap_max, 2048);
+    p.cap = std::min(p.cap, (n_ctx + 63) / 64 * 64);
+    p.S = (n_ctx + p.cap - 1) / p.cap;
+    p.lds = ((size_t) p.cap * p.M + (size_t) G * p.M * rank + 8 * p.M + 8 + 256 * p.M) * 4;
+    p.scratch = (size_t) n_tok * heads * rank * (1 + p.S) + (size_t) n_tok * heads * p.S * 2;
+    return p;
+}
+
+template <int RPT>
+__global__ void __launch_bounds__(256) k_latent_absorb(const float * __restrict__ q, int64_t qs, const uint16_t * __restrict__ wuk, float scale, int heads, int dim, int rank, int n_tok,
+                                                       float * __restrict__ qa, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w, 5)) return;
+    const int t0 = blockIdx.x * 4, h = blockIdx.y, r0 = threadIdx.x * RPT;
+    if (r0 >= rank) return;
+    float acc[4][RPT];
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+        for (int i = 0; i < RPT; i++) acc[tt][i] = 0.0f;
+    const uint16_t * w = wuk + (int64_t) h * dim * rank + r0;
+#pragma unroll 8
+    for (int d = 0; d < dim; d++) {
+        float wv[RPT];
+#pragma unroll
+        for (int i = 0; i < RPT; i++) wv[i] = r0 + i < rank ? hy_widen(w[(int64_t) d * rank + i]) : 0.0f;
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++) {
+            const float qv = q[(int64_t) min(t0 + tt, n_tok - 1) * qs + (int64_t) h * dim + d];
+#pragma unroll
+            for (int i = 0; i < RPT; i++) acc[tt][i] = fmaf(qv, wv[i], acc[tt][i]);
+        }
+    }
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++)
+        if (t0 + tt < n_tok)
+#pragma unroll
+            for (int i = 0; i < RPT; i++) if (r0 + i < rank) qa[((int64_t) (t0 + tt) * heads + h) * rank + r0 + i] = acc[tt][i] * scale;
+}
+
+template <int M, int RPT>
+__global__ void __launch_bounds__(256) k_latent_scores(const float * __restrict__ qa, const float * __restrict__ cache, const uint32_t * __restrict__ mask, int heads, int rank, int n_kv_arg,
+                                                       int cap, int S, float * __restrict__ pol, float * __restrict__ pml, const int32_t * __restrict__ dyn, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
     extern __shared__ float lds[];
-    __shared__ float red[4], hm[HT], hden[HT];
-    const int t = blockIdx.x, h0 = blockIdx.y * HT, nh = min(HT, heads - h0), tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n_kv = min(dyn ? dyn[1] : n_kv_arg, cap);
+    const int t = blockIdx.x, h0 = blockIdx.y * M, split = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int rthreads = (rank + RPT - 1) / RPT, G = max(1, 256 / rthreads);
+    float * sc = lds, * part = sc + (size_t) cap * M, * red = part + (size_t) G * M * rank, * wsc = red + 8 * M + 8;     // red: [4 waves][M] twice; wsc: [4 waves][64 cells][M]
+    __shared__ int hi_s;
+    const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg);
     const int words = (n_kv_arg + 31) / 32;
-    float * qa = lds, * ol = qa + HT * rank, * sc = ol + 4 * HT * rank;
-    for (int idx = tid; idx < nh * rank; idx += 256) {
-        const int hh = idx / rank, r = idx % rank;
-        const float * qh = q + (int64_t) t * qs + (int64_t) (h0 + hh) * dim;
-        const uint16_t * wk = wuk + (int64_t) (h0 + hh) * dim * rank + r;
-        float a = 0.0f;
-        for (int d = 0; d < dim; d++) a = fmaf(qh[d], hy_widen(wk[(int64_t) d * rank]), a);
-        qa[idx] = a * scale;
+    const uint32_t * mrow = mask + (int64_t) t * words;
+    const int c0 = split * cap;
+    int c1 = min(n_kv, c0 + cap);
+    if (tid == 0) hi_s = 0;
+    __syncthreads();
+    {   // cells past the last visible one of this token are not walked (a prompt's early tokens see little of the pass's cells)
+        int hi = 0;
+        for (int w = (c0 >> 5) + tid; w < (c1 + 31) >> 5; w += 256) { const uint32_t bits = mrow[w]; if (bits) hi = max(hi, w * 32 + 32 - __clz(bits)); }
+        if (hi) atomicMax(&hi_s, hi);
     }
     __syncthreads();
-    const uint32_t * mrow = mask + (int64_t) t * words;
-    float lmax[HT];
+    c1 = min(c1, hi_s);
+    const int nh = min(M, heads - h0);
+    const float * qat = qa + ((int64_t) t * heads + h0) * rank;
+    float * pol_t = pol + (((int64_t) t * heads + h0) * S + split) * rank, * pml_t = pml + (((int64_t) t * heads + h0) * S + split) * 2;
+    if (c1 <= c0) {                                                   // nothing of this token lives in this split: an empty partial
+        for (int m = 0; m < nh; m++) {
+            for (int r = tid; r < rank; r += 256) pol_t[(int64_t) m * S * rank + r] = 0.0f;
+            if (tid == 0) { pml_t[(int64_t) m * S * 2] = -INFINITY; pml_t[(int64_t) m * S * 2 + 1] = 0.0f; }
+        }
+        return;
+    }
+    // scores: a thread per cell; a split of 64 cells (single tokens) gives every wave a quarter of the rank instead, so that all four waves stream the 64 latents
+    float lmax[M];
 #pragma unroll
-    for (int hh = 0; hh < HT; hh++) lmax[hh] = -INFINITY;
-    for (int j = tid; j < n_kv; j += 256) {
+    for (int m = 0; m < M; m++) lmax[m] = -INFINITY;
+    if (cap == 64 && (rank & 15) == 0) {
+        const int j = c0 + lane, rq = rank >> 2, rb = wave * rq;
+        const bool vis = j < c1 && ((mrow[j >> 5] >> (j & 31)) & 1u);
+        float a[M];
+#pragma unroll
+        for (int m = 0; m < M; m++) a[m] = 0.0f;
+        if (vis) {
+            const float * c = cache + (int64_t) j * rank + rb;
+#pragma unroll 2
+            for (int r = 0; r < rq; r += 4) {
+                const float4 cv = *(const float4 *) (c + r);
+#pragma unroll
+                for (int m = 0; m < M; m++) {
+                    const float * qq = qat + (m < nh ? m : 0) * rank + rb + r;                    // (wave-uniform address)
+                    a[m] = fmaf(qq[0], cv.x, a[m]); a[m] = fmaf(qq[1], cv.y, a[m]); a[m] = fmaf(qq[2], cv.z, a[m]); a[m] = fmaf(qq[3], cv.w, a[m]);
+                }
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < M; m++) wsc[((size_t) wave * 64 + lane) * M + m] = a[m];
+        __syncthreads();
+        if (wave == 0 && j < c1) {
+#pragma unroll
+            for (int m = 0; m < M; m++) {
+                const float sv = vis ? wsc[(size_t) lane * M + m] + wsc[((size_t) 64 + lane) * M + m] + wsc[((size_t) 128 + lane) * M + m] + wsc[((size_t) 192 + lane) * M + m] : -INFINITY;
+                sc[(size_t) lane * M + m] = sv; lmax[m] = sv;
+            }
+        }
+        __syncthreads();
+    } else
+    for (int j = c0 + tid; j < c1; j += 256) {
         const bool vis = (mrow[j >> 5] >> (j & 31)) & 1u;
-        float a[HT];
+        float a[M];
 #pragma unroll
-        for (int hh = 0; hh < HT; hh++) a[hh] = 0.0f;
+        for (int m = 0; m < M; m++) a[m] = 0.0f;
         if (vis) {
             const float * c = cache + (int64_t) j * rank;
             if ((rank & 3) == 0) {
+#pragma unroll 2
                 for (int r = 0; r < rank; r += 4) {
                     const float4 cv = *(const float4 *) (c + r);
 #pragma unroll
-                    for (int hh = 0; hh < HT; hh++) {
-                        const float * qq = qa + hh * rank + r;
-                        a[hh] = fmaf(qq[0], cv.x, a[hh]); a[hh] = fmaf(qq[1], cv.y, a[hh]); a[hh] = fmaf(qq[2], cv.z, a[hh]); a[hh] = fmaf(qq[3], cv.w, a[hh]);
+                    for (int m = 0; m < M; m++) {
+                        const float * qq = qat + (m < nh ? m : 0) * rank + r;                     // (wave-uniform address)
+                        a[m] = fmaf(qq[0], cv.x, a[m]); a[m] = fmaf(qq[1], cv.y, a[m]); a[m] = fmaf(qq[2], cv.z, a[m]); a[m] = fmaf(qq[3], cv.w, a[m]);
                     }
                 }
             } else {
                 for (int r = 0; r < rank; r++) {
                     const float cv = c[r];
 #pragma unroll
-                    for (int hh = 0; hh < HT; hh++) a[hh] = fmaf(qa[hh * rank + r], cv, a[hh]);
+                    for (int m = 0; m < M; m++) a[m] = fmaf(qat[(m < nh ? m : 0) * rank + r], cv, a[m]);
                 }
             }
         }
 #pragma unroll
-        for (int hh = 0; hh < HT; hh++) {
-            const float s = vis ? a[hh] : -INFINITY;
-            if (hh < nh) sc[hh * cap + j] = s;
-            lmax[hh] = fmaxf(lmax[hh], s);
-        }
+        for (int m = 0; m < M; m++) { const float sv = vis ? a[m] : -INFINITY; sc[(size_t) (j - c0) * M + m] = sv; lmax[m] = fmaxf(lmax[m], sv); }
     }
+    // per head: max over the split, then p = exp(s - max) and its sum (every thread revisits its own cells)
 #pragma unroll
-    for (int hh = 0; hh < HT; hh++) {
-        const float m = hy_block_max(lmax[hh], red);
-        if (tid == 0 && hh < nh) hm[hh] = fmaxf(m, sink[h0 + hh]);
-    }
+    for (int m = 0; m < M; m++) { const float v = pi_wave_max(lmax[m]); if (lane == 0) red[wave * M + m] = v; }
     __syncthreads();
+    float mx[M], lsum[M];
 #pragma unroll
-    for (int hh = 0; hh < HT; hh++) {
-        float l = 0.0f;
-        if (hh < nh) {
-            const float m = hm[hh];
-            for (int j = tid; j < n_kv; j += 256) { const float p = expf(sc[hh * cap + j] - m); sc[hh * cap + j] = p; l += p; }
+    for (int m = 0; m < M; m++) { mx[m] = fmaxf(fmaxf(red[m], red[M + m]), fmaxf(red[2 * M + m], red[3 * M + m])); lsum[m] = 0.0f; }
+    for (int j = c0 + tid; j < c1; j += 256)
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            const float sv = sc[(size_t) (j - c0) * M + m];
+            const float pv = sv == -INFINITY ? 0.0f : expf(sv - mx[m]);
+            sc[(size_t) (j - c0) * M + m] = pv; lsum[m] += pv;
         }
-        l = hy_block_sum(l, red);
-        if (tid == 0 && hh < nh) hden[hh] = l + expf(sink[h0 + hh] - hm[hh]);
-    }
+    float * red2 = red + 4 * M;
+#pragma unroll
+    for (int m = 0; m < M; m++) { const float v = pi_lanes_sum<64>(lsum[m]); if (lane == 0) red2[wave * M + m] = v; }
     __syncthreads();
-    // probability-weighted sum of latents: wave w takes cells w, w + 4, ...; lanes walk the (head, r) pairs
-    for (int base = 0; base < nh * rank; base += 64) {
-        const int idx = base + lane;
-        const bool ok = idx < nh * rank;
-        const int hh = ok ? idx / rank : 0, r = ok ? idx % rank : 0;
-        float a = 0.0f;
-        for (int j = wave; j < n_kv; j += 4) {
-            const float p = sc[hh * cap + j];
-            if (p != 0.0f) a = fmaf(p, cache[(int64_t) j * rank + r], a);
+    if (tid < nh) {
+        pml_t[(int64_t) tid * S * 2] = fmaxf(fmaxf(red[tid], red[M + tid]), fmaxf(red[2 * M + tid], red[3 * M + tid]));
+        pml_t[(int64_t) tid * S * 2 + 1] = red2[tid] + red2[M + tid] + red2[2 * M + tid] + red2[3 * M + tid];
+    }
+    // sum of p * c: thread (cell group g, rank slice rt)
+    const int g = tid / rthreads, rt = tid % rthreads, r0 = rt * RPT;
+    float o[M][RPT];
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+        for (int i = 0; i < RPT; i++) o[m][i] = 0.0f;
+    if (g < G) {
+#pragma unroll 4
+        for (int j = c0 + g; j < c1; j += G) {                          // (a masked cell has p = 0: its latent — zeros or an earlier owner's finite values — adds nothing)
+            float cv[RPT];
+#pragma unroll
+            for (int i = 0; i < RPT; i++) cv[i] = r0 + i < rank ? cache[(int64_t) j * rank + r0 + i] : 0.0f;
+            const float * pj = sc + (size_t) (j - c0) * M;
+#pragma unroll
+            for (int m = 0; m < M; m++) {
+                const float pv = pj[m];
+#pragma unroll
+                for (int i = 0; i < RPT; i++) o[m][i] = fmaf(pv, cv[i], o[m][i]);
+            }
         }
-        if (ok) ol[wave * HT * rank + idx] = a;
+        if (G > 1)
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int i = 0; i < RPT; i++) if (r0 + i < rank) part[((size_t) g * M + m) * rank + r0 + i] = o[m][i];
     }
-    __syncthreads();
-    for (int idx = tid; idx < nh * rank; idx += 256)
-        ol[idx] = (ol[idx] + ol[HT * rank + idx] + ol[2 * HT * rank + idx] + ol[3 * HT * rank + idx]) / hden[idx / rank];
-    __syncthreads();
-    // value up-projection: one wave per output value
-    for (int o = wave; o < nh * vdim; o += 4) {
-        const int hh = o / vdim, vv = o % vdim;
-        const uint16_t * wv = wuv + ((int64_t) (h0 + hh) * vdim + vv) * rank;
-        float a = 0.0f;
-        for (int r = lane; r < rank; r += 64) a = fmaf(hy_widen(wv[r]), ol[hh * rank + r], a);
-        a = pi_lanes_sum<64>(a);
-        if (lane == 0) out[(int64_t) t * os + (int64_t) (h0 + hh) * vdim + vv] = a;
+    if (G > 1) {
+        __syncthreads();
+        for (int idx = tid; idx < nh * rank; idx += 256) {
+            const int m = idx / rank, r = idx % rank;
+            float v = 0.0f;
+            for (int gg = 0; gg < G; gg++) v += part[((size_t) gg * M + m) * rank + r];
+            pol_t[(int64_t) m * S * rank + r] = v;
+        }
+    } else if (g == 0) {
+#pragma unroll
+        for (int m = 0; m < M; m++)
+            if (m < nh)
+#pragma unroll
+                for (int i = 0; i < RPT; i++) if (r0 + i < rank) pol_t[(int64_t) m * S * rank + r0 + i] = o[m][i];
     }
 }
 
-#define LAT_LDS_BUDGET (144 * 1024)
-static int latent_tile(int heads, int rank, int cap, int n_tok) {
-    int ht = n_tok >= 8 ? 8 : 1;                                     // single tokens: one head per workgroup (more workgroups); prompts: the cache row is read once for 8 heads
-    while (ht > 1 && (ht / 2 >= heads || ((size_t) 5 * ht * rank + (size_t) ht * cap) * 4 > LAT_LDS_BUDGET)) ht /= 2;
-    return ht;
+// grid (token tile of 4, head): merges the splits (with the sink), normalises, applies W_uv[h]
+__global__ void __launch_bounds__(256) k_latent_combine(const float * __restrict__ pol, const float * __restrict__ pml, const uint16_t * __restrict__ wuv, const float * __restrict__ sink,
+                                                        int heads, int vdim, int rank, int S, int n_tok, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w, 5)) return;
+    extern __shared__ float ol[];                                     // [4][rank]
+    __shared__ float wgt[4][64 + 1];                                  // per token: weight of every split (S <= 64 at a time), [64]: 1 / denominator
+    const int t0 = blockIdx.x * 4, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nt = min(4, n_tok - t0);
+    for (int idx = tid; idx < 4 * rank; idx += 256) ol[idx] = 0.0f;
+    // (the wave `tt` owns token t0 + tt's bookkeeping)
+    float mstar = -INFINITY, den = 0.0f;
+    const float sk = sink[h];
+    const float * pml_t = pml + ((int64_t) (t0 + min(wave, nt - 1)) * heads + h) * S * 2;
+    {
+        float m = sk;
+        for (int s = lane; s < S; s += 64) m = fmaxf(m, pml_t[s * 2]);
+        mstar = pi_wave_max(m);
+        float d = 0.0f;
+        for (int s = lane; s < S; s += 64) { const float ms = pml_t[s * 2]; if (ms != -INFINITY) d += pml_t[s * 2 + 1] * expf(ms - mstar); }
+        den = pi_lanes_sum<64>(d) + expf(sk - mstar);
+    }
+    for (int sb = 0; sb < S; sb += 64) {
+        __syncthreads();
+        if (wave < nt) {
+            const int s = sb + lane;
+            const float ms = s < S ? pml_t[s * 2] : -INFINITY;
+            wgt[wave][lane] = ms == -INFINITY ? 0.0f : expf(ms - mstar) / den;
+        }
+        __syncthreads();
+        for (int idx = tid; idx < nt * rank; idx += 256) {
+            const int tt = idx / rank, r = idx % rank;
+            const float * p = pol + (((int64_t) (t0 + tt) * heads + h) * S + sb) * rank + r;
+            float v = ol[idx];
+            for (int s = 0; s < min(64, S - sb); s++) { const float w = wgt[tt][s]; if (w != 0.0f) v = fmaf(w, p[(int64_t) s * rank], v); }
+            ol[idx] = v;
+        }
+    }
+    __syncthreads();
+    for (int vv = wave; vv < vdim; vv += 4) {
+        const uint16_t * wv = wuv + ((int64_t) h * vdim + vv) * rank;
+        float a[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+#pragma unroll 4
+        for (int r = lane; r < rank; r += 64) {
+            const float w = hy_widen(wv[r]);
+#pragma unroll
+            for (int tt = 0; tt < 4; tt++) a[tt] = fmaf(w, ol[tt * rank + r], a[tt]);
+        }
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++) { const float v = pi_lanes_sum<64>(a[tt]); if (lane == 0 && tt < nt) out[(int64_t) (t0 + tt) * os + (int64_t) h * vdim + vv] = v; }
+    }
 }
-extern "C" int pi_op_latent_attention_max_cells(int rank) { return (int) std::min<int64_t>(LAT_LDS_BUDGET / 4 - 5 * (int64_t) rank, 1 << 20); }
-extern "C" int pi_op_latent_attention_reserve(void) {
-    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_latent_attention<1>, hipFuncAttributeMaxDynamicSharedMemorySize, LAT_LDS_BUDGET));
-    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_latent_attention<2>, hipFuncAttributeMaxDynamicSharedMemorySize, LAT_LDS_BUDGET));
-    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_latent_attention<4>, hipFuncAttributeMaxDynamicSharedMemorySize, LAT_LDS_BUDGET));
-    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_latent_attention<8>, hipFuncAttributeMaxDynamicSharedMemorySize, LAT_LDS_BUDGET));
+
+extern "C" int pi_op_latent_attention_max_cells(int rank) { (void) rank; return 1 << 22; }       // (long contexts are cut into splits: no score row has to fit LDS whole)
+extern "C" size_t pi_op_latent_attention_scratch_floats(int heads, int rank, int n_tok, int n_ctx) {
+    return std::max(latent_plan(heads, rank, n_tok, n_ctx).scratch, latent_plan(heads, rank, std::min(n_tok, 8), n_ctx).scratch);
+}
+template <int M, int RPT> static int latent_reserve_one() {
+    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_latent_scores<M, RPT>, hipFuncAttributeMaxDynamicSharedMemorySize, LAT_LDS_BUDGET + 4096));
     return 0;
 }
+extern "C" int pi_op_latent_attention_reserve(void) {
+    static bool done = false;
+    if (done) return 0;
+#define LAT_RES(M) if (latent_reserve_one<M, 1>() || latent_reserve_one<M, 2>() || latent_reserve_one<M, 4>()) return -1;
+    LAT_RES(1) LAT_RES(2) LAT_RES(4) LAT_RES(8) LAT_RES(16)
+#undef LAT_RES
+    done = true;
+    return 0;
+}
+template <int M, int RPT>
+static void latent_scores_launch(const lat_plan & p, dim3 grid, hipStream_t s, double bytes, int nta, const float * qa, const float * cache, const uint32_t * mask, int heads, int rank, int n_kv,
+                                 float * pol, float * pml, const int32_t * dyn) {
+    PI_KT_LAUNCH(PI_KT_ATT, PI_BF16, nta, bytes, (k_latent_scores<M, RPT>), grid, dim3(256), p.lds, s, qa, cache, mask, heads, rank, n_kv, p.cap, p.S, pol, pml, dyn, pi_abort_word());
+}
 extern "C" int pi_op_latent_attention(const float * q, int64_t q_stride, const float * cache, const uint32_t * mask, const pi_weight * wuk, const pi_weight * wuv, const float * sink_dev,
-                                      float scale, int heads, int dim, int vdim, int rank, int n_tok, int n_kv, float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
+                                      float scale, int heads, int dim, int vdim, int rank, int n_tok, int n_kv, float * scratch_dev, size_t scratch_floats, float * out, int64_t out_stride,
+                                      const int32_t * dyn_dev, void * stream) {
     if (n_tok <= 0) return 0;
     if (!wuk || !wuv || wuk->type != PI_BF16 || wuv->type != PI_BF16 || wuk->ne0 != rank || wuv->ne0 != rank || wuk->ne1 != (int64_t) heads * dim || wuv->ne1 != (int64_t) heads * vdim) {
         pi_set_error("pi_op_latent_attention: the up-projections must be bfloat16 [heads * dim][rank] and [heads * vdim][rank]"); return -1;
     }
-    if (((size_t) 5 * rank + (size_t) n_kv) * 4 > LAT_LDS_BUDGET) { pi_set_error("pi_op_latent_attention: %d cells of rank %d do not fit a workgroup's score row", n_kv, rank); return -1; }
-    const int ht = latent_tile(heads, rank, n_kv, n_tok);
-    const size_t lds = ((size_t) 5 * ht * rank + (size_t) ht * n_kv) * 4;
-    const dim3 grid((unsigned) n_tok, (unsigned) ((heads + ht - 1) / ht));
-    const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
-    const double bytes = 4.0 * acct * rank + 2.0 * rank * heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim);
+    if (rank > 1024) { pi_set_error("pi_op_latent_attention: latent width %d above 1024", rank); return -1; }
+    const lat_plan p = latent_plan(heads, rank, n_tok, n_kv);
+    if (p.scratch > scratch_floats) { pi_set_error("pi_op_latent_attention: %zu floats of scratch needed, %zu given", p.scratch, scratch_floats); return -1; }
+    if (p.lds > LAT_LDS_BUDGET + 4096 || (size_t) 4 * rank * 4 > 64 * 1024) { pi_set_error("pi_op_latent_attention: LDS plan does not fit"); return -1; }
+    if (pi_op_latent_attention_reserve() != 0) return -1;
     hipStream_t s = (hipStream_t) stream;
-#define LAT_GO(H) PI_KT_LAUNCH(PI_KT_ATT, PI_BF16, std::min(n_tok, PI_KT_MAXNT - 1), bytes, k_latent_attention<H>, grid, dim3(256), lds, s, q, q_stride, cache, mask, (const uint16_t *) wuk->p0, (const uint16_t *) wuv->p0, \
-                                sink_dev, scale, heads, dim, vdim, rank, n_kv, n_kv, out, out_stride, dyn_dev, pi_abort_word())
-    if (ht == 8) LAT_GO(8); else if (ht == 4) LAT_GO(4); else if (ht == 2) LAT_GO(2); else LAT_GO(1);
+    float * qa = scratch_dev, * pol = qa + (size_t) n_tok * heads * rank, * pml = pol + (size_t) n_tok * heads * p.S * rank;
+    const int nta = std::min(n_tok, PI_KT_MAXNT - 1);
+    const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
+    const dim3 ga((unsigned) ((n_tok + 3) / 4), (unsigned) heads);
+#define LAT_ABS(R) PI_KT_LAUNCH(PI_KT_ATT, PI_BF16, nta, 2.0 * rank * heads * dim + 4.0 * n_tok * heads * (dim + rank), k_latent_absorb<R>, ga, dim3(256), 0, s, q, q_stride, (const uint16_t *) wuk->p0, scale, heads, dim, rank, n_tok, qa, pi_abort_word())
+    if (p.RPT == 1) LAT_ABS(1); else if (p.RPT == 2) LAT_ABS(2); else LAT_ABS(4);
+#undef LAT_ABS
+    PI_CHECK_LAUNCH();
+    const dim3 grid((unsigned) n_tok, (unsigned) ((heads + p.M - 1) / p.M), (unsigned) p.S);
+    const double bytes = 4.0 * acct * rank + 4.0 * n_tok * heads * rank * (1.0 + p.S);
+#define LAT_GO(M) do { if (p.RPT == 1) latent_scores_launch<M, 1>(p, grid, s, bytes, nta, qa, cache, mask, heads, rank, n_kv, pol, pml, dyn_dev); \
+                       else if (p.RPT == 2) latent_scores_launch<M, 2>(p, grid, s, bytes, nta, qa, cache, mask, heads, rank, n_kv, pol, pml, dyn_dev); \
+                       else latent_scores_launch<M, 4>(p, grid, s, bytes, nta, qa, cache, mask, heads, rank, n_kv, pol, pml, dyn_dev); } while (0)
+    switch (p.M) { case 16: LAT_GO(16); break; case 8: LAT_GO(8); break; case 4: LAT_GO(4); break; case 2: LAT_GO(2); break; default: LAT_GO(1); }
 #undef LAT_GO
+    PI_CHECK_LAUNCH();
+    PI_KT_LAUNCH(PI_KT_ATT, PI_BF16, nta, 2.0 * rank * heads * vdim + 4.0 * n_tok * heads * (rank * p.S + vdim), k_latent_combine, ga, dim3(256), (size_t) 16 * rank, s,
+                 pol, pml, (const uint16_t *) wuv->p0, sink_dev, heads, vdim, rank, p.S, n_tok, out, out_stride, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
 }
 
 // ---- routed feed-forward ------------------------------------------------------------------------------------------------------------------------------
 // one workgroup per token: logits of all router outputs (a wave per output), soft-max, choice = score + correction, `top` rounds of arg-max (lowest index wins a tie)
 __global__ void __launch_bounds__(256) k_moe_route(const uint16_t * __restrict__ router, int64_t width, int n_out, const float * __restrict__ corr, const float * __restrict__ x, int64_t xs,
-                                                   int top, int exact, int32_t * __restrict__ sel, float * __restrict__ selw, const int32_t * __restrict__ abort_w) {
+                                                   int top, int exact, int vec, int32_t * __restrict__ sel, float * __restrict__ selw, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     extern __shared__ float z[];                  // [n_out] logits -> scores | [n_out] choice
     float * ch = z + n_out;
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float * xr = x + (int64_t) t * xs;
     for (int e = wave; e < n_out; e += 4) {
-        const uint16_t * w = router + (int64_t) e * width;
-        float a = 0.0f;
-        for (int64_t i = lane; i < width; i += 64) a = fmaf(hy_widen(w[i]), exact ? xr[i] : hy_round(xr[i]), a);
-        a = pi_lanes_sum<64>(a);
+        const float a = pi_lanes_sum<64>(hy_dot_lane(router + (int64_t) e * width, xr, width, lane, exact != 0, vec != 0));
         if (lane == 0) z[e] = a;
     }
     __syncthreads();
@@ -342,22 +577,19 @@ __global__ void __launch_bounds__(256) k_moe_route(const uint16_t * __restrict__
 
 // up[t][kk][f] = relu(W_up[e] x_t)^2 for the kk-th chosen expert e of token t (nothing for identity experts); a wave per row f
 __global__ void __launch_bounds__(256) k_moe_up(const uint16_t * __restrict__ wup, int64_t width, int ff, int n_exp, const float * __restrict__ x, int64_t xs, const int32_t * __restrict__ sel,
-                                                int top, int exact, float * __restrict__ up, const int32_t * __restrict__ abort_w) {
+                                                int top, int exact, int vec, float * __restrict__ up, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 0)) return;
     const int lane = threadIdx.x & 63, f = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int slot = blockIdx.y, e = sel[slot];
     if (f >= ff || e >= n_exp) return;
     const int t = slot / top;
     const float * xr = x + (int64_t) t * xs;
-    const uint16_t * w = wup + ((int64_t) e * ff + f) * width;
-    float a = 0.0f;
-    for (int64_t i = lane; i < width; i += 64) a = fmaf(hy_widen(w[i]), exact ? xr[i] : hy_round(xr[i]), a);
-    a = pi_lanes_sum<64>(a);
+    const float a = pi_lanes_sum<64>(hy_dot_lane(wup + ((int64_t) e * ff + f) * width, xr, width, lane, exact != 0, vec != 0));
     if (lane == 0) { const float r = fmaxf(a, 0.0f); up[(int64_t) slot * ff + f] = r * r; }
 }
 // out[t][n] = sum_kk w_kk * (identity ? x[t][n] : W_down[e_kk][n] . up[t][kk]); a wave per output n
 __global__ void __launch_bounds__(256) k_moe_down(const uint16_t * __restrict__ wdown, int64_t width, int ff, int n_exp, int top, const float * __restrict__ x, int64_t xs,
-                                                  const int32_t * __restrict__ sel, const float * __restrict__ selw, const float * __restrict__ up, int exact, float * __restrict__ out, int64_t os,
+                                                  const int32_t * __restrict__ sel, const float * __restrict__ selw, const float * __restrict__ up, int exact, int vec, float * __restrict__ out, int64_t os,
                                                   const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 0)) return;
     const int lane = threadIdx.x & 63;
@@ -369,11 +601,7 @@ __global__ void __launch_bounds__(256) k_moe_down(const uint16_t * __restrict__ 
         const int e = sel[(int64_t) t * top + kk];
         const float wgt = selw[(int64_t) t * top + kk];
         if (e >= n_exp) { acc = fmaf(wgt, x[(int64_t) t * xs + n], acc); continue; }
-        const uint16_t * w = wdown + ((int64_t) e * width + n) * ff;
-        const float * u = up + ((int64_t) t * top + kk) * ff;
-        float a = 0.0f;
-        for (int i = lane; i < ff; i += 64) a = fmaf(hy_widen(w[i]), exact ? u[i] : hy_round(u[i]), a);
-        a = pi_lanes_sum<64>(a);
+        const float a = pi_lanes_sum<64>(hy_dot_lane(wdown + ((int64_t) e * width + n) * ff, up + ((int64_t) t * top + kk) * ff, ff, lane, exact != 0, vec != 0));
         acc = fmaf(wgt, a, acc);
     }
     if (lane == 0) out[(int64_t) t * os + n] = acc;
@@ -383,7 +611,8 @@ extern "C" int pi_op_moe_route(const pi_weight * router, const float * correctio
     if (n_tok <= 0) return 0;
     if (!router || router->type != PI_BF16 || top < 1 || top > router->ne1 || router->ne1 > 8192) { pi_set_error("pi_op_moe_route: a bfloat16 router of at most 8192 outputs and 1 <= top <= outputs are required"); return -1; }
     PI_KT_LAUNCH(PI_KT_OTHER, PI_BF16, 1, 2.0 * router->ne0 * router->ne1 + 4.0 * n_tok * router->ne0, k_moe_route, dim3((unsigned) n_tok), dim3(256), (size_t) 8 * router->ne1, (hipStream_t) stream,
-                 (const uint16_t *) router->p0, router->ne0, (int) router->ne1, correction_dev, x, x_stride, top, exact, sel_dev, selw_dev, pi_abort_word());
+                 (const uint16_t *) router->p0, router->ne0, (int) router->ne1, correction_dev, x, x_stride, top, exact,
+                 (int) (router->ne0 % 8 == 0 && ((uintptr_t) router->p0 % 16) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0), sel_dev, selw_dev, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
 }
 // wup: [n_exp * ff][width], wdown: [n_exp * width][ff] (the experts' matrices one after the other); up_dev: scratch [n_tok][top][ff]
@@ -399,12 +628,14 @@ extern "C" int pi_op_moe_experts(const pi_weight * wup, const pi_weight * wdown,
         width = wup->ne0;
         const double b_up = std::min<double>(n_tok * top, n_exp) * 2.0 * ff * width + 4.0 * n_tok * (width + (double) top * ff);
         PI_KT_LAUNCH(PI_KT_MATVEC, PI_BF16, std::min(n_tok, PI_KT_MAXNT - 1), b_up, k_moe_up, dim3((unsigned) ((ff + 3) / 4), (unsigned) (n_tok * top)), dim3(256), 0, s,
-                     (const uint16_t *) wup->p0, width, ff, n_exp, x, x_stride, sel_dev, top, exact, up_dev, pi_abort_word());
+                     (const uint16_t *) wup->p0, width, ff, n_exp, x, x_stride, sel_dev, top, exact,
+                     (int) (width % 8 == 0 && ((uintptr_t) wup->p0 % 16) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0), up_dev, pi_abort_word());
         PI_CHECK_LAUNCH();
     } else width = out_stride;
     const double b_dn = std::min<double>(n_tok * top, std::max(n_exp, 1)) * 2.0 * ff * width + 4.0 * n_tok * (width + (double) top * ff);
     PI_KT_LAUNCH(PI_KT_MATVEC, PI_BF16, std::min(n_tok, PI_KT_MAXNT - 1), b_dn, k_moe_down, dim3((unsigned) ((width + 3) / 4), (unsigned) n_tok), dim3(256), 0, s,
-                 n_exp > 0 ? (const uint16_t *) wdown->p0 : nullptr, width, ff, n_exp, top, x, x_stride, sel_dev, selw_dev, up_dev, exact, out, out_stride, pi_abort_word());
+                 n_exp > 0 ? (const uint16_t *) wdown->p0 : nullptr, width, ff, n_exp, top, x, x_stride, sel_dev, selw_dev, up_dev, exact,
+                 (int) (n_exp > 0 && ff % 8 == 0 && ((uintptr_t) wdown->p0 % 16) == 0 && ((uintptr_t) up_dev % 16) == 0), out, out_stride, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
 }
 

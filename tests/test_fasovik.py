@@ -289,7 +289,8 @@ def pack_mask(vis, n_kv):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,D,V,R,T,n_kv", [(1, 4, 6, 10, 1, 33), (3, 8, 10, 20, 5, 70), (9, 16, 12, 96, 9, 300), (6, 32, 24, 64, 20, 700), (2, 24, 40, 130, 3, 1500)])
+@pytest.mark.parametrize("H,D,V,R,T,n_kv", [(1, 4, 6, 10, 1, 33), (3, 8, 10, 20, 5, 70), (9, 16, 12, 96, 9, 300), (6, 32, 24, 64, 20, 700), (2, 24, 40, 130, 3, 1500), (16, 8, 8, 300, 12, 2500),
+                                            (5, 8, 8, 520, 2, 200), (17, 4, 4, 32, 33, 90)])
 def test_latent_attention_against_explicit_keys_and_values(H, D, V, R, T, n_kv):
     U, lib = gpu()
     rng = np.random.default_rng(R + T)
@@ -313,7 +314,9 @@ def test_latent_attention_against_explicit_keys_and_values(H, D, V, R, T, n_kv):
         dyn = np.array([0, n_kv, T, 0], np.int32)
         args = [U.Dev(a) for a in (q, cache, pack_mask(vis, n_ctx), sink, dyn)]
         ukd, uvd, od = upload_bf16(lib, wuk), upload_bf16(lib, wuv), U.Dev(nbytes=4 * T * H * V)
-        L.check(lib.pi_op_latent_attention(args[0].ptr, H * D + 7, args[1].ptr, args[2].ptr, ukd, uvd, args[3].ptr, 0.37, H, D, V, R, T, n_ctx, od.ptr, H * V, args[4].ptr, None))
+        nscr = lib.pi_op_latent_attention_scratch_floats(H, R, T, n_ctx)
+        scr = U.Dev(nbytes=4 * nscr)
+        L.check(lib.pi_op_latent_attention(args[0].ptr, H * D + 7, args[1].ptr, args[2].ptr, ukd, uvd, args[3].ptr, 0.37, H, D, V, R, T, n_ctx, scr.ptr, nscr, od.ptr, H * V, args[4].ptr, None))
         got = od.get(np.float32, (T, H * V))
         want = latent_ref(q[:, :H * D].astype(np.float64), np.nan_to_num(cache), vis, wuk.astype(np.float64), wuv.astype(np.float64), sink.astype(np.float64), 0.37, H, D, V)
         assert np.isfinite(got).all() and rel_rms(got, want) < 5e-5, rel_rms(got, want)
@@ -339,7 +342,9 @@ def test_latent_attention_sink_takes_its_share():
         sink = np.full(H, sk, np.float32)
         ukd, uvd, od = upload_bf16(lib, wuk), upload_bf16(lib, wuv), U.Dev(nbytes=4 * H * V)
         a = [U.Dev(x) for x in (q, cache, pack_mask(vis, n), sink, np.array([0, n, 1, 0], np.int32))]
-        L.check(lib.pi_op_latent_attention(a[0].ptr, H * D, a[1].ptr, a[2].ptr, ukd, uvd, a[3].ptr, 0.5, H, D, V, R, 1, n, od.ptr, H * V, a[4].ptr, None))
+        nscr = lib.pi_op_latent_attention_scratch_floats(H, R, 1, n)
+        scr = U.Dev(nbytes=4 * nscr)
+        L.check(lib.pi_op_latent_attention(a[0].ptr, H * D, a[1].ptr, a[2].ptr, ukd, uvd, a[3].ptr, 0.5, H, D, V, R, 1, n, scr.ptr, nscr, od.ptr, H * V, a[4].ptr, None))
         outs.append(od.get(np.float32, (1, H * V)))
         want = latent_ref(q.astype(np.float64), cache, vis, wuk.astype(np.float64), wuv.astype(np.float64), sink.astype(np.float64), 0.5, H, D, V)
         assert rel_rms(outs[-1], want) < 5e-5

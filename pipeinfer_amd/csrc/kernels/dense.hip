@@ -7,7 +7,8 @@
 //
 //   k_dense_rows   one wave per output row, K spread over the lanes with 16 / 8 / 2-byte weight loads, TT tokens held in registers: the mat-vec of decode (weights streamed
 //                  once from HBM whatever TT is) and every width of the fp32 mode
-//   k_dense_mfma   serving precision, >= 16 tokens: 64 tokens x 64 rows per workgroup on v_mfma_f32_16x16x32_bf16; a wave owns 16 tokens and four 16-row tiles, operands go
+//   k_dense_mfma_lds  serving precision, >= 96 tokens: 128 tokens x 128 rows per workgroup, both operands staged through LDS as bfloat16, double-buffered
+//   k_dense_mfma   serving precision, 16 .. 95 tokens: 64 tokens x 64 rows per workgroup on v_mfma_f32_16x16x32_bf16; a wave owns 16 tokens and four 16-row tiles, operands go
 //                  straight from global memory into the lane layout of the instruction (A: weight row l % 16, k block l / 16; B: token l % 16, k block l / 16)
 //   k_embed        rows of the table gathered, widened and scaled
 #include "ops_common.h"
@@ -124,6 +125,82 @@ __global__ void __launch_bounds__(256) k_dense_mfma(const uint16_t * __restrict_
         }
 }
 
+// 128 tokens x 128 rows per workgroup, operands staged through LDS as bfloat16 (activations are rounded once, while they are staged): a wave owns 64 x 64 = sixteen 16 x 16
+// tiles, so one K step of 32 costs it eight 16-byte LDS reads for sixteen MFMAs; the next K step's global loads are in flight while the current one is multiplied.
+// K % 8 == 0, 16-byte aligned rows of W and X.
+__global__ void __launch_bounds__(256) k_dense_mfma_lds(const uint16_t * __restrict__ W, int64_t K, int64_t N, const float * __restrict__ X, int64_t xs, int T, float * __restrict__ Y, int64_t ys,
+                                                        int act_a, int64_t rows_a, int act_b, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w, 1)) return;
+    __shared__ __attribute__((aligned(16))) uint16_t sw[2][128 * 32], sx[2][128 * 32];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+    const int wr = wave >> 1, wt = wave & 1;                           // the wave's 64 rows / 64 tokens inside the tile
+    const int64_t n0 = (int64_t) blockIdx.x * 128;
+    const int t0 = blockIdx.y * 128;
+    // staging: thread -> (row or token tid / 2, 16 k values of half tid % 2)
+    const int sr = tid >> 1, sh = tid & 1;
+    const bool w_ok = n0 + sr < N, x_ok = t0 + sr < T;
+    const uint16_t * wsrc = W + (w_ok ? n0 + sr : 0) * K + sh * 16;
+    const float * xsrc = X + (int64_t) (x_ok ? t0 + sr : 0) * xs + sh * 16;
+    uint4 wreg[2]; float4 xreg[4];
+    auto fetch = [&](int64_t k0) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) wreg[i] = (w_ok && k0 + sh * 16 + i * 8 < K) ? *(const uint4 *) (wsrc + k0 + i * 8) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) xreg[i] = (x_ok && k0 + sh * 16 + i * 4 < K) ? *(const float4 *) (xsrc + k0 + i * 4) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    };
+    auto stage = [&](int buf) {
+        *(uint4 *) (sw[buf] + sr * 32 + sh * 16) = wreg[0]; *(uint4 *) (sw[buf] + sr * 32 + sh * 16 + 8) = wreg[1];
+        uint32_t pk[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            pk[2 * i]     = dn_round_bits(xreg[i].x) | dn_round_bits(xreg[i].y) << 16;
+            pk[2 * i + 1] = dn_round_bits(xreg[i].z) | dn_round_bits(xreg[i].w) << 16;
+        }
+        *(uint4 *) (sx[buf] + sr * 32 + sh * 16) = make_uint4(pk[0], pk[1], pk[2], pk[3]); *(uint4 *) (sx[buf] + sr * 32 + sh * 16 + 8) = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+    };
+    dn_f32x4 acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) acc[a][b] = dn_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    int buf = 0;
+    for (int64_t k0 = 0; k0 < K; k0 += 32) {
+        const bool more = k0 + 32 < K;
+        if (more) fetch(k0 + 32);
+        dn_u16x8 af[4], bf[4];
+#pragma unroll
+        for (int a = 0; a < 4; a++) af[a] = *(const dn_u16x8 *) (sw[buf] + (wr * 64 + a * 16 + li) * 32 + kb * 8);
+#pragma unroll
+        for (int b = 0; b < 4; b++) bf[b] = *(const dn_u16x8 *) (sx[buf] + (wt * 64 + b * 16 + li) * 32 + kb * 8);
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dn_bf16x8, af[a]), __builtin_bit_cast(dn_bf16x8, bf[b]), acc[a][b], 0, 0, 0);
+        if (more) stage(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        const int tok = t0 + wt * 64 + b * 16 + li;
+        if (tok >= T) continue;
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            const int64_t row = n0 + wr * 64 + a * 16 + kb * 4;
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) v[r] = dn_act(acc[a][b][r], row + r < rows_a ? act_a : act_b);
+            float * dst = Y + (int64_t) tok * ys + row;
+            if (row + 3 < N && (ys & 3) == 0 && (((uintptr_t) Y) & 15) == 0) *(float4 *) dst = make_float4(v[0], v[1], v[2], v[3]);
+            else for (int r = 0; r < 4; r++) if (row + r < N) dst[r] = v[r];
+        }
+    }
+}
+
 extern "C" int pi_op_embed(const pi_weight * w, const int32_t * tokens, int n_tok, float scale, float * out, void * stream) {
     if (!w || w->type != PI_BF16) { pi_set_error("pi_op_embed: the table must be a bfloat16 weight"); return -1; }
     if (n_tok <= 0) return 0;
@@ -152,6 +229,12 @@ extern "C" int pi_op_dense(const pi_weight * w, const float * x, int64_t x_strid
     const double bytes = 2.0 * K * w->ne1 + 4.0 * n_tok * (K + w->ne1);
     const bool al16 = K % 8 == 0 && ((uintptr_t) w->p0 % 16) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0;
     const bool al8  = K % 4 == 0 && ((uintptr_t) w->p0 % 8) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0;
+    static const int lds_min = getenv("PI_DENSE_LDS_MIN") ? atoi(getenv("PI_DENSE_LDS_MIN")) : 96;
+    if (!exact && al16 && n_tok >= lds_min) {
+        PI_KT_LAUNCH(PI_KT_MMQ, PI_BF16, std::min(n_tok, PI_KT_MAXNT - 1), bytes, k_dense_mfma_lds, dim3((unsigned) ((w->ne1 + 127) / 128), (unsigned) ((n_tok + 127) / 128)), dim3(256), 0, s,
+                     (const uint16_t *) w->p0, K, w->ne1, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, pi_abort_word());
+        PI_CHECK_LAUNCH(); return 0;
+    }
     if (!exact && al16 && n_tok >= dense_mfma_min_tokens()) {
         PI_KT_LAUNCH(PI_KT_MMQ, PI_BF16, std::min(n_tok, PI_KT_MAXNT - 1), bytes, k_dense_mfma, dim3((unsigned) ((w->ne1 + 63) / 64), (unsigned) ((n_tok + 63) / 64)), dim3(256), 0, s,
                      (const uint16_t *) w->p0, K, w->ne1, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, pi_abort_word());

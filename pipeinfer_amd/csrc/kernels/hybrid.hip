@@ -177,7 +177,9 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
                 for (int ii = 0; ii < DPT; ii++)
                     if (sp * DPT + ii < dim) { S[ii] = fmaf(kr[ii], vj, lam * S[ii]); o = fmaf(S[ii], qr[ii], o); }
             }
-            for (int d = R >> 1; d > 0; d >>= 1) o += __shfl_xor(o, d, PI_WAVE);
+            if (R == 2) o += pi_partner<1>(o);
+            else if (R == 4) { o += pi_partner<2>(o); o += pi_partner<1>(o); }
+            else for (int d = R >> 1; d > 0; d >>= 1) o += __shfl_xor(o, d, PI_WAVE);
             if (col_ok && sp == 0) out[(int64_t) (first + t0 + tt) * os + (int64_t) h * vdim + j] = o;
         }
     }
@@ -190,7 +192,7 @@ extern "C" int pi_op_linear_attention(const float * q, const float * k, const fl
                                       const int32_t * rec_dev, int n_tok, int max_segments, float * out, int64_t out_stride, void * stream) {
     if (n_tok <= 0) return 0;
     if (dim <= 0 || vdim <= 0 || heads <= 0 || dim > 1024) { pi_set_error("pi_op_linear_attention: head sizes %d x %d outside the kernel's range (key width <= 1024)", dim, vdim); return -1; }
-    const int dpt = dim <= 16 ? 16 : dim <= 32 ? 32 : 64;
+    const int dpt = dim <= 8 ? 8 : dim <= 16 ? 16 : 32;                // state values a thread keeps in registers (more would spill in the token loop)
     int R = 1; while (R * dpt < dim) R *= 2;
     int threads = std::min(256, (vdim * R + 63) / 64 * 64);
     const int cols = threads / R;
@@ -199,7 +201,7 @@ extern "C" int pi_op_linear_attention(const float * q, const float * k, const fl
     const double bytes = 4.0 * n_tok * heads * (2.0 * dim + 2.0 * vdim) + 8.0 * heads * dim * vdim;
     hipStream_t s = (hipStream_t) stream;
 #define LA_GO(D) PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), bytes, k_linear_attention<D>, grid, dim3(threads), lds, s, q, k, v, stride, heads, dim, vdim, R, decay_dev, state_dev, rec_dev, n_tok, out, out_stride, pi_abort_word())
-    if (dpt == 16) LA_GO(16); else if (dpt == 32) LA_GO(32); else LA_GO(64);
+    if (dpt == 8) LA_GO(8); else if (dpt == 16) LA_GO(16); else LA_GO(32);
 #undef LA_GO
     PI_CHECK_LAUNCH(); return 0;
 }
@@ -241,35 +243,26 @@ static lat_plan latent_plan(int heads, int rank, int n_tok, int n_ctx) {
     return p;
 }
 
-template <int RPT>
+// grid (token tile of 4, head, 64 values of the rank): lane = one rank value, the four waves take a quarter of the head's dim each and meet in LDS
 __global__ void __launch_bounds__(256) k_latent_absorb(const float * __restrict__ q, int64_t qs, const uint16_t * __restrict__ wuk, float scale, int heads, int dim, int rank, int n_tok,
                                                        float * __restrict__ qa, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
-    const int t0 = blockIdx.x * 4, h = blockIdx.y, r0 = threadIdx.x * RPT;
-    if (r0 >= rank) return;
-    float acc[4][RPT];
-#pragma unroll
-    for (int tt = 0; tt < 4; tt++)
-#pragma unroll
-        for (int i = 0; i < RPT; i++) acc[tt][i] = 0.0f;
-    const uint16_t * w = wuk + (int64_t) h * dim * rank + r0;
+    __shared__ float part[4][4][64];
+    const int t0 = blockIdx.x * 4, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = blockIdx.z * 64 + lane;
+    const int dq = (dim + 3) / 4, d0 = wave * dq, d1 = min(dim, d0 + dq);
+    float acc[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+    const uint16_t * w = wuk + (int64_t) h * dim * rank + min(r, rank - 1);
 #pragma unroll 8
-    for (int d = 0; d < dim; d++) {
-        float wv[RPT];
+    for (int d = d0; d < d1; d++) {
+        const float wv = hy_widen(w[(int64_t) d * rank]);
 #pragma unroll
-        for (int i = 0; i < RPT; i++) wv[i] = r0 + i < rank ? hy_widen(w[(int64_t) d * rank + i]) : 0.0f;
-#pragma unroll
-        for (int tt = 0; tt < 4; tt++) {
-            const float qv = q[(int64_t) min(t0 + tt, n_tok - 1) * qs + (int64_t) h * dim + d];
-#pragma unroll
-            for (int i = 0; i < RPT; i++) acc[tt][i] = fmaf(qv, wv[i], acc[tt][i]);
-        }
+        for (int tt = 0; tt < 4; tt++) acc[tt] = fmaf(q[(int64_t) min(t0 + tt, n_tok - 1) * qs + (int64_t) h * dim + d], wv, acc[tt]);
     }
 #pragma unroll
-    for (int tt = 0; tt < 4; tt++)
-        if (t0 + tt < n_tok)
-#pragma unroll
-            for (int i = 0; i < RPT; i++) if (r0 + i < rank) qa[((int64_t) (t0 + tt) * heads + h) * rank + r0 + i] = acc[tt][i] * scale;
+    for (int tt = 0; tt < 4; tt++) part[wave][tt][lane] = acc[tt];
+    __syncthreads();
+    const int tt = wave;                                              // wave tt writes token t0 + tt
+    if (t0 + tt < n_tok && r < rank) qa[((int64_t) (t0 + tt) * heads + h) * rank + r] = (part[0][tt][lane] + part[1][tt][lane] + part[2][tt][lane] + part[3][tt][lane]) * scale;
 }
 
 template <int M, int RPT>
@@ -433,7 +426,7 @@ __global__ void __launch_bounds__(256) k_latent_scores(const float * __restrict_
     }
 }
 
-// grid (token tile of 4, head): merges the splits (with the sink), normalises, applies W_uv[h]
+// grid (token tile of 4, head, 16 output values): merges the splits (with the sink), normalises, applies its rows of W_uv[h]
 __global__ void __launch_bounds__(256) k_latent_combine(const float * __restrict__ pol, const float * __restrict__ pml, const uint16_t * __restrict__ wuv, const float * __restrict__ sink,
                                                         int heads, int vdim, int rank, int S, int n_tok, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
@@ -471,7 +464,7 @@ __global__ void __launch_bounds__(256) k_latent_combine(const float * __restrict
         }
     }
     __syncthreads();
-    for (int vv = wave; vv < vdim; vv += 4) {
+    for (int vv = blockIdx.z * 16 + wave; vv < min(vdim, (int) blockIdx.z * 16 + 16); vv += 4) {
         const uint16_t * wv = wuv + ((int64_t) h * vdim + vv) * rank;
         float a[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
 #pragma unroll 4
@@ -523,10 +516,8 @@ extern "C" int pi_op_latent_attention(const float * q, int64_t q_stride, const f
     float * qa = scratch_dev, * pol = qa + (size_t) n_tok * heads * rank, * pml = pol + (size_t) n_tok * heads * p.S * rank;
     const int nta = std::min(n_tok, PI_KT_MAXNT - 1);
     const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
-    const dim3 ga((unsigned) ((n_tok + 3) / 4), (unsigned) heads);
-#define LAT_ABS(R) PI_KT_LAUNCH(PI_KT_ATT, PI_BF16, nta, 2.0 * rank * heads * dim + 4.0 * n_tok * heads * (dim + rank), k_latent_absorb<R>, ga, dim3(256), 0, s, q, q_stride, (const uint16_t *) wuk->p0, scale, heads, dim, rank, n_tok, qa, pi_abort_word())
-    if (p.RPT == 1) LAT_ABS(1); else if (p.RPT == 2) LAT_ABS(2); else LAT_ABS(4);
-#undef LAT_ABS
+    PI_KT_LAUNCH(PI_KT_ATT, PI_BF16, nta, 2.0 * rank * heads * dim + 4.0 * n_tok * heads * (dim + rank), k_latent_absorb, dim3((unsigned) ((n_tok + 3) / 4), (unsigned) heads, (unsigned) ((rank + 63) / 64)), dim3(256), 0, s,
+                 q, q_stride, (const uint16_t *) wuk->p0, scale, heads, dim, rank, n_tok, qa, pi_abort_word());
     PI_CHECK_LAUNCH();
     const dim3 grid((unsigned) n_tok, (unsigned) ((heads + p.M - 1) / p.M), (unsigned) p.S);
     const double bytes = 4.0 * acct * rank + 4.0 * n_tok * heads * rank * (1.0 + p.S);
@@ -536,7 +527,7 @@ extern "C" int pi_op_latent_attention(const float * q, int64_t q_stride, const f
     switch (p.M) { case 16: LAT_GO(16); break; case 8: LAT_GO(8); break; case 4: LAT_GO(4); break; case 2: LAT_GO(2); break; default: LAT_GO(1); }
 #undef LAT_GO
     PI_CHECK_LAUNCH();
-    PI_KT_LAUNCH(PI_KT_ATT, PI_BF16, nta, 2.0 * rank * heads * vdim + 4.0 * n_tok * heads * (rank * p.S + vdim), k_latent_combine, ga, dim3(256), (size_t) 16 * rank, s,
+    PI_KT_LAUNCH(PI_KT_ATT, PI_BF16, nta, 2.0 * rank * heads * vdim + 4.0 * n_tok * heads * (rank * p.S + vdim), k_latent_combine, dim3((unsigned) ((n_tok + 3) / 4), (unsigned) heads, (unsigned) ((vdim + 15) / 16)), dim3(256), (size_t) 16 * rank, s,
                  pol, pml, (const uint16_t *) wuv->p0, sink_dev, heads, vdim, rank, p.S, n_tok, out, out_stride, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
 }

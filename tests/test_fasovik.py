@@ -167,7 +167,7 @@ def upload_bf16(lib, w):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("K,N,T", [(40, 37, 1), (33, 10, 3), (512, 70, 5), (1024, 130, 8), (96, 200, 17), (64, 64, 64), (520, 33, 150)])
+@pytest.mark.parametrize("K,N,T", [(40, 37, 1), (33, 10, 3), (512, 70, 5), (1024, 130, 8), (96, 200, 17), (64, 64, 64), (520, 33, 150), (256, 300, 200), (72, 130, 129)])
 @pytest.mark.parametrize("exact", [True, False])
 def test_dense_every_kernel_and_width(K, N, T, exact):
     U, lib = gpu()

@@ -10,6 +10,8 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG)
 SO = os.environ.get("PIPEINFER_LIB") or os.path.join(PKG, "libpipeinfer_amd.so")        # (override: A/B runs of two builds on one box, tools_dev/)
 
+SO_DENSE = os.path.join(PKG, "libpipeinfer_amd_dense.so")     # `make dense`: the engine with the dense-weight kernels only (hybrid safetensors models need no more)
+
 _lib = None
 
 
@@ -24,8 +26,17 @@ def build(force=False):
     return SO
 
 
-def _stale():
-    t = os.path.getmtime(SO)
+def build_dense():
+    """the library a model of dense bfloat16 weights needs, where the full one is not there: the engine + the dense / hybrid kernels (a fraction of the full build's time)"""
+    if os.path.exists(SO) and not _stale():
+        return SO
+    if not os.path.exists(SO_DENSE) or _stale(SO_DENSE):
+        subprocess.check_call(["make", "-C", os.path.join(PKG, "csrc"), "-j8", "dense"], stdout=subprocess.DEVNULL)
+    return SO_DENSE
+
+
+def _stale(so=None):
+    t = os.path.getmtime(so or SO)
     for d in (os.path.join(PKG, "csrc", "kernels"), os.path.join(PKG, "csrc", "engine"), os.path.join(ROOT, "include")):
         if os.path.isdir(d):
             for f in os.listdir(d):
@@ -49,15 +60,16 @@ def declared_symbols():
     return sorted(set(names))
 
 
-def load():
+def load(dense_ok=False):
+    """dense_ok: the caller only runs dense-weight (safetensors) models, so where the full library is missing the dense-only build will do"""
     global _lib
     if _lib is None:
+        so = SO
         if not os.path.exists(SO):
-            if os.path.exists("/opt/rocm/bin/hipcc"):
-                build()
-            else:
+            if not os.path.exists("/opt/rocm/bin/hipcc") and not (dense_ok and os.path.exists(SO_DENSE)):
                 raise PipeInferError(f"{SO} is missing and hipcc is not available: the MI355X path has no fallback")
-        lib = C.CDLL(SO)
+            so = build_dense() if dense_ok else build()
+        lib = C.CDLL(so)
         _declare(lib)
         _lib = lib
     return _lib

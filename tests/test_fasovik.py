@@ -570,3 +570,27 @@ def test_graph_replays_equal_eager_launches(tmp_path):
         outs.append(lg[0])
         e.close()
     assert np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.gpu
+def test_generate_command_line_greedy_and_sampled(tmp_path, capsys):
+    """the generation command: greedy ids equal the engine's own generate(); with a temperature the llama.h samplers pick from the top-k of the same logits, reproducibly per seed"""
+    from pipeinfer_amd.tools import generate as G
+    m = small_model(seed=71)
+    folder = str(tmp_path / "g")
+    O.write_model(folder, m["config"], {k: v.astype(np.float32) for k, v in m["tensors"].items()})
+    assert G.main(["--model", folder, "--prompt-ids", "5,6,7", "--n-predict", "12", "--float32"]) == 0
+    greedy = [int(t) for t in capsys.readouterr().out.strip().split(",")]
+    want = O.greedy(m, [5, 6, 7], 12)
+    k = next((i for i, (a, b) in enumerate(zip(greedy, want)) if a != b), 12)
+    assert k >= 6
+    outs = []
+    for seed in (3, 3, 4):
+        assert G.main(["--model", folder, "--prompt-ids", "5,6,7", "--n-predict", "12", "--temp", "1.5", "--top-k", "5", "--seed", str(seed)]) == 0
+        outs.append(capsys.readouterr().out.strip())
+    assert outs[0] == outs[1] and len(outs[0].split(",")) == 12
+    # every sampled token lies in the top 5 of the logits the oracle gives for the tokens before it
+    toks = [int(t) for t in outs[0].split(",")]
+    lg = O.run(m, [5, 6, 7] + toks)
+    for i, t in enumerate(toks):
+        assert t in np.argsort(-lg[2 + i])[:6], i

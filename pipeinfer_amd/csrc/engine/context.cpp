@@ -40,7 +40,7 @@ llama_context::~llama_context() {
     if (hop_host) (void) hipHostFree(hop_host);
     pi_free(hop_dev);
     pi_free(abort_dev);
-    void * bufs[] = { lat_cache, rec_state, rec_dev, h_in, h_att, h_out, moe_w, moe_up, moe_dn, lat_scratch, moe_sel, moe_idx, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
+    void * bufs[] = { lat_cache, rec_state, rec_dev, h_in, h_att, h_out, moe_w, moe_up, moe_dn, lat_scratch, rec_scratch, moe_sel, moe_idx, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
     for (void * b : bufs) pi_free(b);
     if (rope) pi_rope_table_free(rope);
     if (stream) (void) hipStreamDestroy(stream);
@@ -111,11 +111,11 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
             ctx->lat_off[i] = lat; lat += (size_t) ctx->n_ctx * H.kv_rank;
             ctx->lat_scratch_floats = std::max(ctx->lat_scratch_floats, pi_op_latent_attention_scratch_floats(H.heads, H.kv_rank, nb, ctx->n_ctx));
         }
-        if (H.state_index >= 0) { ctx->rec_off[i] = rec; rec += (size_t) ctx->slots->size() * H.heads * H.dim * H.vdim; }
+        if (H.state_index >= 0) { ctx->rec_off[i] = rec; rec += (size_t) ctx->slots->size() * H.heads * H.dim * H.vdim; ctx->rec_scratch_floats = std::max(ctx->rec_scratch_floats, pi_op_linear_attention_scratch_floats(H.heads, H.dim, H.vdim, nb, ctx->slots->size())); }
         in_w = std::max(in_w, (size_t) H.in_rows()); att_w = std::max(att_w, (size_t) H.heads * H.vdim);
         if (H.has_mlp) { up_w = std::max(up_w, (size_t) H.top * std::max(H.ff, 1)); sel_w = std::max(sel_w, (size_t) H.top); idx_n = std::max(idx_n, pi_op_moe_grouped_index_ints(nb, H.top, H.n_expert)); }
     }
-    if (!(ctx->lat_scratch = (float *) dev(ctx->lat_scratch_floats * 4)) || !(ctx->lat_cache = (float *) dev(lat * 4)) || !(ctx->rec_state = (float *) dev(rec * 4))) return false;
+    if (!(ctx->rec_scratch = (float *) dev(ctx->rec_scratch_floats * 4)) || !(ctx->lat_scratch = (float *) dev(ctx->lat_scratch_floats * 4)) || !(ctx->lat_cache = (float *) dev(lat * 4)) || !(ctx->rec_state = (float *) dev(rec * 4))) return false;
     pi_memset(ctx->lat_cache, 0, std::max<size_t>(lat * 4, 16), nullptr); pi_memset(ctx->rec_state, 0, std::max<size_t>(rec * 4, 16), nullptr);
     if (!(ctx->x = (float *) dev((size_t) 4 * nb * width)) || !(ctx->nx = (float *) dev((size_t) 4 * nb * width)) || !(ctx->h_out = (float *) dev((size_t) 4 * nb * width)) ||
         !(ctx->h_in = (float *) dev((size_t) 4 * nb * in_w)) || !(ctx->h_att = (float *) dev((size_t) 4 * nb * att_w)) || !(ctx->moe_up = (float *) dev((size_t) 4 * nb * up_w)) ||
@@ -296,7 +296,7 @@ static bool forward_hybrid(llama_context * ctx, int n_tok, int n_kv) {
         } else {
             float * state = ctx->rec_state + ctx->rec_off[il];
             OP_OK(pi_op_dense(W.w_in, x, width, n_tok, P, pw, PI_ACT_SILU, 2 * hd + hv, PI_ACT_SIGMOID, ex, s));                                   // silu(q | k | v) | sigmoid(g)
-            OP_OK(pi_op_linear_attention(P, P + hd, P + 2 * hd, pw, H.heads, H.dim, H.vdim, W.decay, state, ctx->rec_dev, n_tok, ctx->slots->size(), A, hv, s));
+            OP_OK(pi_op_linear_attention(P, P + hd, P + 2 * hd, pw, H.heads, H.dim, H.vdim, W.decay, state, ctx->rec_dev, n_tok, ctx->slots->size(), ctx->rec_scratch, ctx->rec_scratch_floats, A, hv, s));
             OP_OK(pi_op_rms_scale(A, hv, W.mix_norm, 0.0f, eps, (int) hv, n_tok, P + 2 * hd + hv, pw, nullptr, 0, 1.0f, A, hv, nullptr, 0, s));    // norm over all heads, * gate
         }
         trace(ctx, "mix", (int) il, A, hv, n_tok);

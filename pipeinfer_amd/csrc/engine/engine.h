@@ -188,7 +188,7 @@ struct llama_context {
     std::unique_ptr<pi::state_slots> slots; int n_state_slots = 8;
     int32_t * rec_dev = nullptr;                              // per token of the pass: state slot (| 1 << 30: start from zero)
     int exact = 0;                                            // 1: dense operators keep fp32 activations (pipeinfer_context_set_precision)
-    float * h_in = nullptr, * h_att = nullptr, * h_out = nullptr, * moe_w = nullptr, * moe_up = nullptr, * moe_dn = nullptr, * lat_scratch = nullptr; size_t lat_scratch_floats = 0; int32_t * moe_sel = nullptr, * moe_idx = nullptr;   // hybrid scratch
+    float * h_in = nullptr, * h_att = nullptr, * h_out = nullptr, * moe_w = nullptr, * moe_up = nullptr, * moe_dn = nullptr, * lat_scratch = nullptr, * rec_scratch = nullptr; size_t lat_scratch_floats = 0, rec_scratch_floats = 0; int32_t * moe_sel = nullptr, * moe_idx = nullptr;   // hybrid scratch
     void * rope = nullptr;
     hipStream_t stream = nullptr;
     int stream_priority = 0;                 // > 0 high, < 0 low (pipeinfer_context_set_priority, before the first decode)

@@ -103,44 +103,63 @@ extern "C" int pi_op_rms_scale(const float * x, int64_t x_stride, const float * 
 
 // ---- linear attention with a per-head decay -------------------------------------------------------------------------------------------------------
 // rec[t] = state slot of token t (| 1 << 30 on the first token of a sequence whose state starts from zero), tokens of one slot are consecutive.  Workgroup (head, column block,
-// segment ordinal): thread (column j, part sp of R) keeps S[i][j] for its DPT rows i in registers, walks the segment's tokens in order and leaves S in HBM.
-#define LA_TB 32                                  // tokens whose q, k and v are staged in LDS at a time
+// piece): thread (column j, part sp of R) keeps S[i][j] for its DPT rows i in registers and walks the piece's tokens in order.
+// A pass of up to LA_TB tokens is one launch: a piece is a sequence's whole run, S comes from and goes back to HBM.  Longer passes cut every sequence's run into pieces of LA_TB
+// tokens and take three launches, so that the serial depth is two pieces instead of the whole prompt (the recurrence is linear in S):
+//   mode 1  every piece but a run's last: the state it would build from ZERO, L_p = sum_j lambda^(len-1-j) k_j v_j^T, into scratch
+//   k_linear_state_scan  per run, piece by piece: S_in(p + 1) = lambda^len_p * S_in(p) + L_p, S_in(0) = the slot's state (or zero); scratch[p] <- S_in(p)
+//   mode 2  every piece from its true S_in(p): outputs; a run's last piece leaves the slot's new state
+#define LA_TB 32                                  // tokens of a piece; q, k and v of a piece are staged in LDS
 #define LA_FRESH (1 << 30)
+// finds piece number `want` of the pass (lseg = 0: pieces are whole runs): first token, length, slot word, whether it is its run's last piece
+static __device__ __forceinline__ bool la_find_piece(const int * recs, int n_tok, int lseg, int want, int & first, int & len, int & word, int & last) {
+    int ord = 0, t = 0;
+    while (t < n_tok) {
+        const int sl = recs[t] & ~LA_FRESH;
+        int e = t;
+        while (e < n_tok && (recs[e] & ~LA_FRESH) == sl) e++;
+        const int nsub = lseg > 0 ? (e - t + lseg - 1) / lseg : 1;
+        if (want < ord + nsub) {
+            const int p = want - ord;
+            first = lseg > 0 ? t + p * lseg : t; len = lseg > 0 ? min(lseg, e - first) : e - t; word = recs[t]; last = p == nsub - 1;
+            return true;
+        }
+        ord += nsub; t = e;
+    }
+    return false;
+}
 template <int DPT>
 __global__ void __launch_bounds__(256) k_linear_attention(const float * __restrict__ q, const float * __restrict__ k, const float * __restrict__ v, int64_t stride, int heads, int dim, int vdim, int R,
-                                                          const float * __restrict__ decay, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
+                                                          const float * __restrict__ decay, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, int mode, float * __restrict__ scratch,
                                                           float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     extern __shared__ float lds[];                // q tile [LA_TB][dim] | k tile [LA_TB][dim] | v tile [LA_TB][cols] | the slot words of the pass [n_tok]
-    __shared__ int seg[3];                        // first token, length, slot word
+    __shared__ int seg[4];                        // first token, length, slot word, last piece of its run
     const int h = blockIdx.x, tid = threadIdx.x;
     int * recs = (int *) (lds + 2 * LA_TB * dim + LA_TB * (blockDim.x / R));
     for (int t = tid; t < n_tok; t += blockDim.x) recs[t] = rec[t];
     __syncthreads();
     if (tid == 0) {
-        int ord = -1, first = 0, len = 0, word = -1, prev = -1;
-        for (int t = 0; t < n_tok; t++) {
-            const int s = recs[t] & ~LA_FRESH;
-            if (t == 0 || s != prev) { if (ord == (int) blockIdx.z) break; ord++; first = t; len = 0; word = recs[t]; }
-            prev = s; len++;
-        }
-        if (ord != (int) blockIdx.z) len = 0;
-        seg[0] = first; seg[1] = len; seg[2] = word;
+        int first = 0, len = 0, word = -1, last = 1;
+        if (!la_find_piece(recs, n_tok, mode ? LA_TB : 0, blockIdx.z, first, len, word, last)) len = 0;
+        seg[0] = first; seg[1] = len; seg[2] = word; seg[3] = last;
     }
     __syncthreads();
-    const int first = seg[0], len = seg[1], word = seg[2];
-    if (len == 0 || word < 0) return;
+    const int first = seg[0], len = seg[1], word = seg[2], last = seg[3];
+    if (len == 0 || word < 0 || (mode == 1 && last)) return;
     const int slot = word & ~LA_FRESH;
     const int cols = blockDim.x / R;
     const int j = blockIdx.y * cols + tid / R, sp = tid % R;
     const bool col_ok = j < vdim;
     const float lam = decay[h];
     float * S_hbm = state + ((int64_t) slot * heads + h) * dim * vdim;
+    float * S_scr = scratch ? scratch + ((int64_t) blockIdx.z * heads + h) * dim * vdim : nullptr;
+    const float * S_from = mode == 2 ? S_scr : mode == 1 || (word & LA_FRESH) ? nullptr : S_hbm;
     float S[DPT];
 #pragma unroll
     for (int ii = 0; ii < DPT; ii++) {
         const int i = sp * DPT + ii;
-        S[ii] = (col_ok && i < dim && !(word & LA_FRESH)) ? S_hbm[(int64_t) i * vdim + j] : 0.0f;
+        S[ii] = (col_ok && i < dim && S_from) ? S_from[(int64_t) i * vdim + j] : 0.0f;
     }
     float * qt = lds, * kt = lds + LA_TB * dim, * vt = kt + LA_TB * dim;
     const bool dim4 = (dim & 3) == 0;
@@ -150,13 +169,23 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
         for (int idx = tid; idx < nt * dim; idx += blockDim.x) {
             const int tt = idx / dim, i = idx % dim;
             const int64_t off = (int64_t) (first + t0 + tt) * stride + (int64_t) h * dim + i;
-            qt[idx] = q[off]; kt[idx] = k[off];
+            if (mode != 1) qt[idx] = q[off];
+            kt[idx] = k[off];
         }
         for (int idx = tid; idx < nt * cols; idx += blockDim.x) {
             const int tt = idx / cols, jj = blockIdx.y * cols + idx % cols;
             vt[idx] = jj < vdim ? v[(int64_t) (first + t0 + tt) * stride + (int64_t) h * vdim + jj] : 0.0f;
         }
         __syncthreads();
+        if (mode == 1) {                                              // the state only
+            for (int tt = 0; tt < nt; tt++) {
+                const float vj = vt[tt * cols + tid / R];
+                const float * kr = kt + tt * dim + sp * DPT;
+#pragma unroll
+                for (int ii = 0; ii < DPT; ii++) if (sp * DPT + ii < dim) S[ii] = fmaf(kr[ii], vj, lam * S[ii]);
+            }
+            continue;
+        }
         for (int tt = 0; tt < nt; tt++) {
             const float vj = vt[tt * cols + tid / R];
             const float * kr = kt + tt * dim + sp * DPT, * qr = qt + tt * dim + sp * DPT;
@@ -183,25 +212,76 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
             if (col_ok && sp == 0) out[(int64_t) (first + t0 + tt) * os + (int64_t) h * vdim + j] = o;
         }
     }
-    if (col_ok)
+    float * S_to = mode == 1 ? S_scr : last ? S_hbm : nullptr;
+    if (col_ok && S_to)
 #pragma unroll
-        for (int ii = 0; ii < DPT; ii++) { const int i = sp * DPT + ii; if (i < dim) S_hbm[(int64_t) i * vdim + j] = S[ii]; }
+        for (int ii = 0; ii < DPT; ii++) { const int i = sp * DPT + ii; if (i < dim) S_to[(int64_t) i * vdim + j] = S[ii]; }
 }
 
+// grid (head, blocks over dim * vdim, run): scratch[piece] holds L_p coming in and S_in(p) going out
+__global__ void __launch_bounds__(256) k_linear_state_scan(int heads, int dim, int vdim, const float * __restrict__ decay, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
+                                                           float * __restrict__ scratch, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    __shared__ int seg[3];                        // slot word, first piece ordinal, pieces of the run (0: no such run)
+    if (threadIdx.x == 0) {
+        int ord = 0, t = 0, run = 0, nsub = 0, word = -1, sub0 = 0;
+        while (t < n_tok) {
+            const int sl = rec[t] & ~LA_FRESH;
+            int e = t;
+            while (e < n_tok && (rec[e] & ~LA_FRESH) == sl) e++;
+            const int ns = (e - t + LA_TB - 1) / LA_TB;
+            if (run == (int) blockIdx.z) { nsub = ns; word = rec[t]; sub0 = ord; break; }
+            ord += ns; t = e; run++;
+        }
+        seg[0] = word; seg[1] = sub0; seg[2] = nsub;
+    }
+    __syncthreads();
+    const int word = seg[0], sub0 = seg[1], nsub = seg[2];
+    if (nsub == 0 || word < 0) return;
+    const int h = blockIdx.x, slot = word & ~LA_FRESH;
+    const int64_t per = (int64_t) dim * vdim, idx = (int64_t) blockIdx.y * 256 + threadIdx.x;
+    if (idx >= per) return;
+    float lp = 1.0f;                                                   // lambda^LA_TB: every piece but a run's last has LA_TB tokens
+    for (int i = 0; i < LA_TB; i++) lp *= decay[h];
+    float run = (word & LA_FRESH) ? 0.0f : state[((int64_t) slot * heads + h) * per + idx];
+    for (int p = 0; p < nsub; p++) {
+        float * cell = scratch + ((int64_t) (sub0 + p) * heads + h) * per + idx;
+        const float lpart = p < nsub - 1 ? *cell : 0.0f;
+        *cell = run;
+        run = fmaf(lp, run, lpart);
+    }
+}
+
+static int la_max_pieces(int n_tok, int max_segments) { return n_tok / LA_TB + std::min(n_tok, std::max(1, max_segments)) + 1; }
+extern "C" size_t pi_op_linear_attention_scratch_floats(int heads, int dim, int vdim, int n_tok, int max_segments) {
+    return n_tok <= LA_TB ? 0 : (size_t) la_max_pieces(n_tok, max_segments) * heads * dim * vdim;
+}
 extern "C" int pi_op_linear_attention(const float * q, const float * k, const float * v, int64_t stride, int heads, int dim, int vdim, const float * decay_dev, float * state_dev,
-                                      const int32_t * rec_dev, int n_tok, int max_segments, float * out, int64_t out_stride, void * stream) {
+                                      const int32_t * rec_dev, int n_tok, int max_segments, float * scratch_dev, size_t scratch_floats, float * out, int64_t out_stride, void * stream) {
     if (n_tok <= 0) return 0;
     if (dim <= 0 || vdim <= 0 || heads <= 0 || dim > 1024) { pi_set_error("pi_op_linear_attention: head sizes %d x %d outside the kernel's range (key width <= 1024)", dim, vdim); return -1; }
     const int dpt = dim <= 8 ? 8 : dim <= 16 ? 16 : 32;                // state values a thread keeps in registers (more would spill in the token loop)
     int R = 1; while (R * dpt < dim) R *= 2;
     int threads = std::min(256, (vdim * R + 63) / 64 * 64);
     const int cols = threads / R;
-    const dim3 grid((unsigned) heads, (unsigned) ((vdim + cols - 1) / cols), (unsigned) std::max(1, std::min(n_tok, max_segments)));
+    const bool pieces = n_tok > LA_TB;
+    if (pieces && (!scratch_dev || scratch_floats < pi_op_linear_attention_scratch_floats(heads, dim, vdim, n_tok, max_segments))) { pi_set_error("pi_op_linear_attention: a pass of %d tokens needs %zu floats of scratch", n_tok, pi_op_linear_attention_scratch_floats(heads, dim, vdim, n_tok, max_segments)); return -1; }
+    const unsigned gz = pieces ? (unsigned) la_max_pieces(n_tok, max_segments) : (unsigned) std::max(1, std::min(n_tok, max_segments));
+    const dim3 grid((unsigned) heads, (unsigned) ((vdim + cols - 1) / cols), gz);
     const size_t lds = ((size_t) 2 * LA_TB * dim + (size_t) LA_TB * cols + (size_t) n_tok) * sizeof(float);
     const double bytes = 4.0 * n_tok * heads * (2.0 * dim + 2.0 * vdim) + 8.0 * heads * dim * vdim;
     hipStream_t s = (hipStream_t) stream;
-#define LA_GO(D) PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), bytes, k_linear_attention<D>, grid, dim3(threads), lds, s, q, k, v, stride, heads, dim, vdim, R, decay_dev, state_dev, rec_dev, n_tok, out, out_stride, pi_abort_word())
-    if (dpt == 8) LA_GO(8); else if (dpt == 16) LA_GO(16); else LA_GO(32);
+    const int nta = std::min(n_tok, PI_KT_MAXNT - 1);
+#define LA_GO(D, MODE) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, bytes, k_linear_attention<D>, grid, dim3(threads), lds, s, q, k, v, stride, heads, dim, vdim, R, decay_dev, state_dev, rec_dev, n_tok, MODE, scratch_dev, out, out_stride, pi_abort_word())
+#define LA_ANY(MODE) do { if (dpt == 8) LA_GO(8, MODE); else if (dpt == 16) LA_GO(16, MODE); else LA_GO(32, MODE); } while (0)
+    if (!pieces) { LA_ANY(0); PI_CHECK_LAUNCH(); return 0; }
+    LA_ANY(1);
+    PI_CHECK_LAUNCH();
+    PI_KT_LAUNCH(PI_KT_ATT, 0, nta, 12.0 * gz * heads * dim * vdim, k_linear_state_scan, dim3((unsigned) heads, (unsigned) (((int64_t) dim * vdim + 255) / 256), (unsigned) std::max(1, std::min(n_tok, max_segments))), dim3(256), 0, s,
+                 heads, dim, vdim, decay_dev, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word());
+    PI_CHECK_LAUNCH();
+    LA_ANY(2);
+#undef LA_ANY
 #undef LA_GO
     PI_CHECK_LAUNCH(); return 0;
 }

@@ -142,7 +142,8 @@ def _declare(lib):
     lib.pi_op_embed.argtypes = [vp, vp, i32, f32, vp, vp]
     lib.pi_op_dense.argtypes = [vp, vp, i64, i32, vp, i64, i32, i64, i32, i32, vp]
     lib.pi_op_rms_scale.argtypes = [vp, i64, vp, f32, f32, i32, i32, vp, i64, vp, i64, f32, vp, i64, vp, i32, vp]
-    lib.pi_op_linear_attention.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp, vp, vp, i32, i32, vp, i64, vp]
+    lib.pi_op_linear_attention.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp, vp, vp, i32, i32, vp, sz, vp, i64, vp]
+    lib.pi_op_linear_attention_scratch_floats.argtypes = [i32, i32, i32, i32, i32]; lib.pi_op_linear_attention_scratch_floats.restype = sz
     lib.pi_op_copy_f32.argtypes = [vp, vp, i64, vp]
     lib.pi_op_latent_attention.argtypes = [vp, i64, vp, vp, vp, vp, vp, f32, i32, i32, i32, i32, i32, i32, vp, sz, vp, i64, vp, vp]
     lib.pi_op_latent_attention_scratch_floats.argtypes = [i32, i32, i32, i32]; lib.pi_op_latent_attention_scratch_floats.restype = sz

@@ -328,15 +328,21 @@ __global__ void __launch_bounds__(256) k_latent_absorb(const float * __restrict_
                                                        float * __restrict__ qa, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
     __shared__ float part[4][4][64];
+    extern __shared__ float4 qsh[];                                    // [dim]: the head's query values of the four tokens, side by side
     const int t0 = blockIdx.x * 4, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = blockIdx.z * 64 + lane;
+    for (int idx = threadIdx.x; idx < 4 * dim; idx += 256) {
+        const int tt = idx / dim, d = idx % dim;
+        ((float *) qsh)[d * 4 + tt] = q[(int64_t) min(t0 + tt, n_tok - 1) * qs + (int64_t) h * dim + d];
+    }
+    __syncthreads();
     const int dq = (dim + 3) / 4, d0 = wave * dq, d1 = min(dim, d0 + dq);
     float acc[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
     const uint16_t * w = wuk + (int64_t) h * dim * rank + min(r, rank - 1);
 #pragma unroll 8
     for (int d = d0; d < d1; d++) {
         const float wv = hy_widen(w[(int64_t) d * rank]);
-#pragma unroll
-        for (int tt = 0; tt < 4; tt++) acc[tt] = fmaf(q[(int64_t) min(t0 + tt, n_tok - 1) * qs + (int64_t) h * dim + d], wv, acc[tt]);
+        const float4 qv = qsh[d];
+        acc[0] = fmaf(qv.x, wv, acc[0]); acc[1] = fmaf(qv.y, wv, acc[1]); acc[2] = fmaf(qv.z, wv, acc[2]); acc[3] = fmaf(qv.w, wv, acc[3]);
     }
 #pragma unroll
     for (int tt = 0; tt < 4; tt++) part[wave][tt][lane] = acc[tt];
@@ -390,7 +396,7 @@ __global__ void __launch_bounds__(256) k_latent_scores(const float * __restrict_
         for (int m = 0; m < M; m++) a[m] = 0.0f;
         if (vis) {
             const float * c = cache + (int64_t) j * rank + rb;
-#pragma unroll 2
+#pragma unroll 8
             for (int r = 0; r < rq; r += 4) {
                 const float4 cv = *(const float4 *) (c + r);
 #pragma unroll
@@ -470,7 +476,7 @@ __global__ void __launch_bounds__(256) k_latent_scores(const float * __restrict_
 #pragma unroll
         for (int i = 0; i < RPT; i++) o[m][i] = 0.0f;
     if (g < G) {
-#pragma unroll 4
+#pragma unroll 8
         for (int j = c0 + g; j < c1; j += G) {                          // (a masked cell has p = 0: its latent — zeros or an earlier owner's finite values — adds nothing)
             float cv[RPT];
 #pragma unroll
@@ -539,7 +545,8 @@ __global__ void __launch_bounds__(256) k_latent_combine(const float * __restrict
             const int tt = idx / rank, r = idx % rank;
             const float * p = pol + (((int64_t) (t0 + tt) * heads + h) * S + sb) * rank + r;
             float v = ol[idx];
-            for (int s = 0; s < min(64, S - sb); s++) { const float w = wgt[tt][s]; if (w != 0.0f) v = fmaf(w, p[(int64_t) s * rank], v); }
+#pragma unroll 8
+            for (int s = 0; s < min(64, S - sb); s++) v = fmaf(wgt[tt][s], p[(int64_t) s * rank], v);                 // (an empty split: weight 0, partial written as zeros)
             ol[idx] = v;
         }
     }
@@ -596,7 +603,7 @@ extern "C" int pi_op_latent_attention(const float * q, int64_t q_stride, const f
     float * qa = scratch_dev, * pol = qa + (size_t) n_tok * heads * rank, * pml = pol + (size_t) n_tok * heads * p.S * rank;
     const int nta = std::min(n_tok, PI_KT_MAXNT - 1);
     const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
-    PI_KT_LAUNCH(PI_KT_ATT, PI_BF16, nta, 2.0 * rank * heads * dim + 4.0 * n_tok * heads * (dim + rank), k_latent_absorb, dim3((unsigned) ((n_tok + 3) / 4), (unsigned) heads, (unsigned) ((rank + 63) / 64)), dim3(256), 0, s,
+    PI_KT_LAUNCH(PI_KT_ATT, PI_BF16, nta, 2.0 * rank * heads * dim + 4.0 * n_tok * heads * (dim + rank), k_latent_absorb, dim3((unsigned) ((n_tok + 3) / 4), (unsigned) heads, (unsigned) ((rank + 63) / 64)), dim3(256), (size_t) 16 * dim, s,
                  q, q_stride, (const uint16_t *) wuk->p0, scale, heads, dim, rank, n_tok, qa, pi_abort_word());
     PI_CHECK_LAUNCH();
     const dim3 grid((unsigned) n_tok, (unsigned) ((heads + p.M - 1) / p.M), (unsigned) p.S);

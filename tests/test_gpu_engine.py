@@ -395,7 +395,7 @@ def test_three_processes_on_one_gpu_through_the_library_transport(tmp_path, tgt,
     # device-side arrival flags (the default in device mode): every run is announced downstream before it is computed and the consuming stage's run is enqueued behind a
     # device-side wait; the flag written by the producing stage's STREAM (behind its peer store) is seen by the waiting kernel within microseconds — no host thread on the
     # critical path of a stage boundary (the reference: blocking MPI_Recv, ggml-mpi.c:451-487)
-    if mode == "probe-fail":
+    if mode == "probe-fail" and "the control block cannot be mapped for device access" not in r.stderr:      # (where the box already publishes from the host, no probe runs that could be made to fail)
         assert "hop probe FAILED" in r.stderr and "Headers are published by the host" in r.stderr
     for s in v["stages"]:
         # decided and logged at the transport's set-up, per rank: how the hop's store is done and what memory the stage's own ring is (round 5: fine-grained by default)

@@ -111,20 +111,32 @@ extern "C" int pi_op_rms_scale(const float * x, int64_t x_stride, const float * 
 //   mode 2  every piece from its true S_in(p): outputs; a run's last piece leaves the slot's new state
 #define LA_TB 32                                  // tokens of a piece; q, k and v of a piece are staged in LDS
 #define LA_FRESH (1 << 30)
-// finds piece number `want` of the pass (lseg = 0: pieces are whole runs): first token, length, slot word, whether it is its run's last piece
-static __device__ __forceinline__ bool la_find_piece(const int * recs, int n_tok, int lseg, int want, int & first, int & len, int & word, int & last) {
-    int ord = 0, t = 0;
-    while (t < n_tok) {
-        const int sl = recs[t] & ~LA_FRESH;
-        int e = t;
-        while (e < n_tok && (recs[e] & ~LA_FRESH) == sl) e++;
+#define LA_MAXRUNS 256                            // sequences a pass may carry (the host checks)
+// the first tokens of the pass's runs, in order (every thread of the block calls; bnd / nb in LDS): a thread looks at its own tokens only, one thread sorts the few it found
+static __device__ __forceinline__ int la_runs(const int * recs, int n_tok, int * bnd, int * nb) {
+    if (threadIdx.x == 0) *nb = 0;
+    __syncthreads();
+    for (int t = threadIdx.x; t < n_tok; t += blockDim.x)
+        if (t == 0 || (recs[t] & ~LA_FRESH) != (recs[t - 1] & ~LA_FRESH)) { const int k = atomicAdd(nb, 1); if (k < LA_MAXRUNS) bnd[k] = t; }
+    __syncthreads();
+    const int n = min(*nb, LA_MAXRUNS);
+    if (threadIdx.x == 0)
+        for (int i = 1; i < n; i++) { const int v = bnd[i]; int j = i - 1; while (j >= 0 && bnd[j] > v) { bnd[j + 1] = bnd[j]; j--; } bnd[j + 1] = v; }
+    __syncthreads();
+    return n;
+}
+// piece number `want` of the pass (lseg = 0: pieces are whole runs): first token, length, slot word, whether it is its run's last piece
+static __device__ __forceinline__ bool la_find_piece(const int * recs, int n_tok, const int * bnd, int n_runs, int lseg, int want, int & first, int & len, int & word, int & last) {
+    int ord = 0;
+    for (int r = 0; r < n_runs; r++) {
+        const int t = bnd[r], e = r + 1 < n_runs ? bnd[r + 1] : n_tok;
         const int nsub = lseg > 0 ? (e - t + lseg - 1) / lseg : 1;
         if (want < ord + nsub) {
             const int p = want - ord;
             first = lseg > 0 ? t + p * lseg : t; len = lseg > 0 ? min(lseg, e - first) : e - t; word = recs[t]; last = p == nsub - 1;
             return true;
         }
-        ord += nsub; t = e;
+        ord += nsub;
     }
     return false;
 }
@@ -134,14 +146,15 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
                                                           float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     extern __shared__ float lds[];                // q tile [LA_TB][dim] | k tile [LA_TB][dim] | v tile [LA_TB][cols] | the slot words of the pass [n_tok]
-    __shared__ int seg[4];                        // first token, length, slot word, last piece of its run
+    __shared__ int seg[4], bnd[LA_MAXRUNS], nbnd; // seg: first token, length, slot word, last piece of its run
     const int h = blockIdx.x, tid = threadIdx.x;
     int * recs = (int *) (lds + 2 * LA_TB * dim + LA_TB * (blockDim.x / R));
     for (int t = tid; t < n_tok; t += blockDim.x) recs[t] = rec[t];
     __syncthreads();
+    const int n_runs = la_runs(recs, n_tok, bnd, &nbnd);
     if (tid == 0) {
         int first = 0, len = 0, word = -1, last = 1;
-        if (!la_find_piece(recs, n_tok, mode ? LA_TB : 0, blockIdx.z, first, len, word, last)) len = 0;
+        if (!la_find_piece(recs, n_tok, bnd, n_runs, mode ? LA_TB : 0, blockIdx.z, first, len, word, last)) len = 0;
         seg[0] = first; seg[1] = len; seg[2] = word; seg[3] = last;
     }
     __syncthreads();
@@ -222,16 +235,18 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
 __global__ void __launch_bounds__(256) k_linear_state_scan(int heads, int dim, int vdim, const float * __restrict__ decay, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
                                                            float * __restrict__ scratch, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
-    __shared__ int seg[3];                        // slot word, first piece ordinal, pieces of the run (0: no such run)
+    __shared__ int seg[3], bnd[LA_MAXRUNS], nbnd; // seg: slot word, first piece ordinal, pieces of the run (0: no such run)
+    extern __shared__ int recs[];                 // the slot words of the pass
+    for (int t = threadIdx.x; t < n_tok; t += 256) recs[t] = rec[t];
+    __syncthreads();
+    const int n_runs = la_runs(recs, n_tok, bnd, &nbnd);
     if (threadIdx.x == 0) {
-        int ord = 0, t = 0, run = 0, nsub = 0, word = -1, sub0 = 0;
-        while (t < n_tok) {
-            const int sl = rec[t] & ~LA_FRESH;
-            int e = t;
-            while (e < n_tok && (rec[e] & ~LA_FRESH) == sl) e++;
+        int ord = 0, nsub = 0, word = -1, sub0 = 0;
+        for (int r = 0; r < n_runs; r++) {
+            const int t = bnd[r], e = r + 1 < n_runs ? bnd[r + 1] : n_tok;
             const int ns = (e - t + LA_TB - 1) / LA_TB;
-            if (run == (int) blockIdx.z) { nsub = ns; word = rec[t]; sub0 = ord; break; }
-            ord += ns; t = e; run++;
+            if (r == (int) blockIdx.z) { nsub = ns; word = recs[t]; sub0 = ord; break; }
+            ord += ns;
         }
         seg[0] = word; seg[1] = sub0; seg[2] = nsub;
     }
@@ -244,11 +259,13 @@ __global__ void __launch_bounds__(256) k_linear_state_scan(int heads, int dim, i
     float lp = 1.0f;                                                   // lambda^LA_TB: every piece but a run's last has LA_TB tokens
     for (int i = 0; i < LA_TB; i++) lp *= decay[h];
     float run = (word & LA_FRESH) ? 0.0f : state[((int64_t) slot * heads + h) * per + idx];
-    for (int p = 0; p < nsub; p++) {
-        float * cell = scratch + ((int64_t) (sub0 + p) * heads + h) * per + idx;
-        const float lpart = p < nsub - 1 ? *cell : 0.0f;
-        *cell = run;
-        run = fmaf(lp, run, lpart);
+    for (int p0 = 0; p0 < nsub; p0 += 8) {                             // eight pieces at a time: their loads are in flight together, then the chain runs on registers
+        float lpart[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) lpart[i] = p0 + i < nsub - 1 ? scratch[((int64_t) (sub0 + p0 + i) * heads + h) * per + idx] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            if (p0 + i < nsub) { scratch[((int64_t) (sub0 + p0 + i) * heads + h) * per + idx] = run; run = fmaf(lp, run, lpart[i]); }
     }
 }
 
@@ -260,6 +277,7 @@ extern "C" int pi_op_linear_attention(const float * q, const float * k, const fl
                                       const int32_t * rec_dev, int n_tok, int max_segments, float * scratch_dev, size_t scratch_floats, float * out, int64_t out_stride, void * stream) {
     if (n_tok <= 0) return 0;
     if (dim <= 0 || vdim <= 0 || heads <= 0 || dim > 1024) { pi_set_error("pi_op_linear_attention: head sizes %d x %d outside the kernel's range (key width <= 1024)", dim, vdim); return -1; }
+    if (max_segments > LA_MAXRUNS) { pi_set_error("pi_op_linear_attention: at most %d sequences in a pass", LA_MAXRUNS); return -1; }
     const int dpt = dim <= 8 ? 8 : dim <= 16 ? 16 : 32;                // state values a thread keeps in registers (more would spill in the token loop)
     int R = 1; while (R * dpt < dim) R *= 2;
     int threads = std::min(256, (vdim * R + 63) / 64 * 64);
@@ -277,7 +295,7 @@ extern "C" int pi_op_linear_attention(const float * q, const float * k, const fl
     if (!pieces) { LA_ANY(0); PI_CHECK_LAUNCH(); return 0; }
     LA_ANY(1);
     PI_CHECK_LAUNCH();
-    PI_KT_LAUNCH(PI_KT_ATT, 0, nta, 12.0 * gz * heads * dim * vdim, k_linear_state_scan, dim3((unsigned) heads, (unsigned) (((int64_t) dim * vdim + 255) / 256), (unsigned) std::max(1, std::min(n_tok, max_segments))), dim3(256), 0, s,
+    PI_KT_LAUNCH(PI_KT_ATT, 0, nta, 12.0 * gz * heads * dim * vdim, k_linear_state_scan, dim3((unsigned) heads, (unsigned) (((int64_t) dim * vdim + 255) / 256), (unsigned) std::max(1, std::min(n_tok, max_segments))), dim3(256), (size_t) 4 * n_tok, s,
                  heads, dim, vdim, decay_dev, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word());
     PI_CHECK_LAUNCH();
     LA_ANY(2);

@@ -190,9 +190,14 @@ llama_model * load_hybrid_model(const std::string & folder, const llama_model_pa
         }
         hp.hybrid.push_back(std::move(H));
     }
+    for (int i = 0; i < hp.n_layer; i++) {                                   // (a borrowed layer may itself borrow: follow to the layer that owns the tensors)
+        int w = hp.hybrid[(size_t) i].weights, hops = 0;
+        while (hp.hybrid[(size_t) w].weights != w && hops++ <= hp.n_layer) w = hp.hybrid[(size_t) w].weights;
+        if (hp.hybrid[(size_t) w].weights != w) return fail("layers[" + std::to_string(i) + "]: 'weights_of' runs in a circle");
+        hp.hybrid[(size_t) i].weights = w;
+    }
     for (int i = 0; i < hp.n_layer; i++) {                                   // a layer that borrows tensors must be the same kind of layer with the same sizes
         const pi_hybrid_layer & a = hp.hybrid[(size_t) i], & b = hp.hybrid[(size_t) a.weights];
-        if (b.weights != a.weights) return fail("layers[" + std::to_string(i) + "]: 'weights_of' names a layer that has no tensors of its own");
         if (a.mixer != b.mixer || a.heads != b.heads || a.dim != b.dim || a.vdim != b.vdim || a.kv_rank != b.kv_rank || a.has_mlp != b.has_mlp || a.n_expert != b.n_expert || a.n_identity != b.n_identity || a.ff != b.ff)
             return fail("layers[" + std::to_string(i) + "]: its sizes differ from those of the layer whose tensors it uses");
     }

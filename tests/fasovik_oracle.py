@@ -160,7 +160,10 @@ def step(model, seq, token, layers_out=None):
     eps, m = cfg["norm"]["eps"], cfg["residual_mult"]
     x = T["embed"][token] * cfg["embedding"]["scale"]
     for i, L in enumerate(cfg["layers"]):
-        p = "l%d." % L.get("weights_of", i)
+        j = i
+        while "weights_of" in cfg["layers"][j]:               # (a borrowed layer may itself borrow)
+            j = cfg["layers"][j]["weights_of"]
+        p = "l%d." % j
         if L["type"] == "lightning":
             y = lightning_step(T, p, L["mixer"], eps, x, seq.per_layer[i])
         elif L["type"] == "latent_attention":

@@ -401,7 +401,7 @@ VARIANTS = {
                     layer("latent_attention", 5, 4, 12, rank=33, scale=0.25, mlp=None),
                     layer("lightning", 4, 5, 17, mlp=None),
                     layer("latent_attention", 1, 6, 5, rank=9, scale=0.9, mlp={"ff": 16, "experts": 3, "identity": 3, "top": 4}, weights_of=1)],
-    "only_lightning": [layer("lightning", 3, 6, 9, mlp=MOE), layer("lightning", 3, 6, 9, mlp=MOE, weights_of=2), layer("lightning", 3, 6, 9, mlp=None)],      # (tensors of a LATER layer)
+    "only_lightning": [layer("lightning", 3, 6, 9, mlp=None), layer("lightning", 3, 6, 9, mlp=MOE, weights_of=2), layer("lightning", 3, 6, 9, mlp=MOE)],      # (tensors of a LATER layer)
     "only_latent": [layer("latent_attention", 5, 6, 4, rank=14, mlp=None), layer("latent_attention", 2, 10, 12, rank=24, scale=0.5, mlp=MOE),
                     layer("latent_attention", 2, 10, 12, rank=24, scale=0.5, mlp=MOE, weights_of=1), layer("latent_attention", 2, 10, 12, rank=24, scale=0.5, mlp=MOE, weights_of=2)],
     "only_identity": [layer("latent_attention", 2, 8, 8, rank=12, mlp={"ff": 0, "experts": 0, "identity": 3, "top": 2}),

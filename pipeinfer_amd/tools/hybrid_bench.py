@@ -110,16 +110,22 @@ def measure(lib, path, n_prompt, n_decode, hybrid, exact=False):
     ctx.feed(toks[n_prompt:n_prompt + 2], n_prompt, 0)
     ctx.seq_rm(0, -1, -1)
     t_pre = []
+    ctx.reset_stats()
     for _ in range(3):
         L.check(lib.pi_device_sync()); t0 = time.perf_counter()
         ctx.feed(toks[:n_prompt], 0, 0)
         t_pre.append(time.perf_counter() - t0)
         if _ < 2:
             ctx.seq_rm(0, -1, -1)
+    st = ctx.stats()
+    res["prefill_gpu_ms"] = round(st["gpu_ms"] / max(1, st["n_calls"]), 3)       # the pass on the GPU (graph replay + the logits' way to the host), without this script's copies
+    ctx.reset_stats()
     t0 = time.perf_counter()
     for i in range(n_decode):
         ctx.feed(toks[n_prompt + i:n_prompt + i + 1], n_prompt + i, 0)
     t_dec = time.perf_counter() - t0
+    st = ctx.stats()
+    res["decode_gpu_ms_per_token"] = round(st["gpu_ms"] / max(1, st["n_calls"]), 4)
     res["prefill_tok_s"] = round(n_prompt / sorted(t_pre)[1], 1)
     res["decode_tok_s"] = round(n_decode / t_dec, 1)
     res["prefill_ms"] = round(sorted(t_pre)[1] * 1e3, 3)

@@ -600,3 +600,32 @@ def test_generate_command_line_greedy_and_sampled(tmp_path, capsys):
     lg = O.run(m, [5, 6, 7] + toks)
     for i, t in enumerate(toks):
         assert t in np.argsort(-lg[2 + i])[:6], i
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_trace_runner_replays_steps_and_writes_the_wanted_rows(tmp_path, dtype):
+    """bin/trace_run as a program: requests one after the other, portions of changing size, rows only where asked, a line per step; against the oracle"""
+    import subprocess
+    import sys
+    m = small_model(seed=81, layers=VARIANTS["other_sizes"], width=40)
+    folder, out = str(tmp_path / "model"), str(tmp_path / "out")
+    O.write_model(folder, m["config"], {k: v.astype(np.float32) for k, v in m["tensors"].items()})
+    rng = np.random.default_rng(5)
+    a, b = [int(t) for t in rng.integers(0, 97, 41)], [int(t) for t in rng.integers(0, 97, 9)]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:3], "want": [0, 2]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[3:33], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[33:40], "want": [6, 1]}], "end": []},
+             {"step": 3, "entries": [{"id": "a", "tokens": a[40:], "want": [0]}], "end": ["a"]},
+             {"step": 4, "entries": [{"id": "b", "tokens": b, "want": [8]}], "end": ["b"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", out, "--max-tokens", "48", "--n-batch", "16"],
+                       input="".join(json.dumps(x) + "\n" for x in steps), capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done %d" % i for i in range(5)]
+    la, lb = O.run(m, a), O.run(m, b)
+    want = {0: la[[0, 2]], 2: la[[39, 34]], 3: la[[40]], 4: lb[[8]]}
+    assert sorted(os.listdir(out)) == sorted("%d.f32" % k for k in want)
+    for k, w in want.items():
+        got = np.fromfile(os.path.join(out, "%d.f32" % k), "<f4").reshape(-1, 97)
+        assert got.shape == w.shape and logit_err(got, w).max() < TOL[dtype == "float32"], k

@@ -293,7 +293,7 @@ def pack_mask(vis, n_kv):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("H,D,V,R,T,n_kv", [(1, 4, 6, 10, 1, 33), (3, 8, 10, 20, 5, 70), (9, 16, 12, 96, 9, 300), (6, 32, 24, 64, 20, 700), (2, 24, 40, 130, 3, 1500), (16, 8, 8, 300, 12, 2500),
-                                            (5, 8, 8, 520, 2, 200), (17, 4, 4, 32, 33, 90)])
+                                            (5, 8, 8, 520, 2, 200), (17, 4, 4, 32, 33, 90), (3, 8, 8, 48, 2, 4500)])
 def test_latent_attention_against_explicit_keys_and_values(H, D, V, R, T, n_kv):
     U, lib = gpu()
     rng = np.random.default_rng(R + T)

@@ -210,10 +210,59 @@ PI_API int pi_op_moe_experts(const pi_weight * w_up, const pi_weight * w_down, i
                              int exact, float * up_dev, float * out_dev, int64_t out_stride, void * stream);
 /* the same result for a prompt's worth of tokens, serving precision: the (token, choice) slots are sorted by expert on the device and every expert's run goes through the
  * matrix cores 64 slots at a time.  up_dev: [n_tok * top][ff], dn_dev: [n_tok * top][width], idx_dev: pi_op_moe_grouped_index_ints(n_tok, top, n_exp) int32 */
-PI_API int pi_op_moe_grouped_ok(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, int n_tok, int top, int exact);
+PI_API int pi_op_moe_grouped_ok(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, int glu, int n_tok, int top, int exact);
 PI_API size_t pi_op_moe_grouped_index_ints(int n_tok, int top, int n_exp);
 PI_API int pi_op_moe_experts_grouped(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, const float * x_dev, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
                                      float * up_dev, float * dn_dev, int32_t * idx_dev, float * out_dev, int64_t out_stride, void * stream);
+
+/* ---- operators of blocks with pre- and post-norms, a learned average over depth, and a mixer of two branches (chunked sigmoid attention beside a selective recurrence) ---- */
+/* y = LayerNorm(ca * a + cb * b) * w + bias (b nullable: one input; the variance is the mean of squared deviations, eps inside the root); out = [residual +] y */
+PI_API int pi_op_layer_norm_mix(const float * a_dev, int64_t a_stride, float ca, const float * b_dev, int64_t b_stride, float cb, const float * w_dev, const float * bias_dev, float eps, int n, int n_tok,
+                                const float * residual_dev, int64_t residual_stride, float * out_dev, int64_t out_stride, void * stream);
+/* out[t] = sum_j coef[j] * hist[j][t], j = 0 .. n_hist - 1 in this order; hist: n_hist arrays of n_tok rows of n floats, hist_stride floats apart; coef_dev: fp32 [n_hist] */
+PI_API int pi_op_depth_mix(const float * hist_dev, int64_t hist_stride, int n_hist, const float * coef_dev, int n, int n_tok, float * out_dev, int64_t out_stride, void * stream);
+/* x <- cap * tanh(x / cap), in place */
+PI_API int pi_op_softcap(float * x_dev, int64_t n, float cap, void * stream);
+/* out[t][f] = in[t][f] * in[t][ff + f] */
+PI_API int pi_op_glu_mul(const float * in_dev, int64_t in_stride, int ff, int n_tok, float * out_dev, int64_t out_stride, void * stream);
+/* pi_op_linear_attention with its options: qk_heads query / key heads shared by heads / qk_heads neighbouring heads each; tdecay_dev / tscale_dev (nullable): fp32 [n_tok][heads]
+ * rows t_stride floats apart, S <- tdecay[t][h] * S + tscale[t][h] * k v^T (tdecay replaces decay_dev); skip_dev (nullable, [heads]): o += skip[h] * v */
+PI_API int pi_op_linear_attention_ex(const float * q_dev, const float * k_dev, const float * v_dev, int64_t stride, int heads, int qk_heads, int dim, int vdim, const float * decay_dev, const float * tdecay_dev,
+                                     const float * tscale_dev, int64_t t_stride, const float * skip_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int max_segments, float * scratch_dev,
+                                     size_t scratch_floats, float * out_dev, int64_t out_stride, void * stream);
+/* cos / sin of p * base^(-2i / dims), p < n_pos, i < dims / 2 (angles formed in double precision on the host) */
+PI_API void * pi_rotary_table_create(int n_pos, int dims, float base);
+PI_API int    pi_rotary_table_positions(const void * table);
+PI_API void   pi_rotary_table_free(void * table);
+/* per token: q and k heads RMS-normed over dim with a weight shared by the heads (eps inside the root), then their first `dims` dimensions rotated by the token's position (dimension i
+ * pairs with i + dims / 2); v heads divided by their root mean square.  q goes to q_out, k and v to the token's cell of k_cache [cells][kv_heads * dim] / v_cache [cells][kv_heads * vdim]
+ * (fp32), and cell_pos_dev [cells] learns the cell's position.  q / k / v rows are `stride` floats apart; dyn_dev as for pi_op_attention_ex */
+PI_API int pi_op_qkv_prepare(const float * q_dev, const float * k_dev, const float * v_dev, int64_t stride, const float * q_norm_w, const float * k_norm_w, float eps, int heads, int kv_heads, int dim, int vdim,
+                             const void * rotary_table, const int32_t * pos_dev, int n_tok, float * q_out_dev, int64_t q_out_stride, float * k_cache_dev, float * v_cache_dev, int32_t * cell_pos_dev,
+                             const int32_t * dyn_dev, void * stream);
+/* out[t][h] = gate[t][h] * sum over the cells c that token t sees of sigmoid(q[t][h] . K[c][h / (heads / kv_heads)] * scale + head_bias[h]) * V[c][..]: no soft-max, no normalisation.
+ * A cell is seen when its bit of the pass's mask is set AND (chunk > 0) its position is not below the start of the chunk of `chunk` positions that holds the token's position.
+ * head_bias_dev, gate_dev nullable (0 and 1); gate_act: PI_ACT_SIGMOID when the gate values are still raw */
+PI_API int pi_op_chunk_attention(const float * q_dev, int64_t q_stride, const float * k_cache_dev, const float * v_cache_dev, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
+                                 const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, int chunk, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv,
+                                 float * out_dev, int64_t out_stride, const int32_t * dyn_dev, void * stream);
+/* out[t][c] = act(bias[c] + sum_l w[c][l] * input(t - (taps - 1 - l))[c]) over the tokens of each sequence (rec_dev as for pi_op_linear_attention); inputs from before the pass come from
+ * state_dev [slots][taps - 1][channels] (oldest first; zeros for a sequence that starts), which then takes the sequence's last taps - 1 inputs.  w_dev: fp32 [channels][taps] */
+PI_API int pi_op_causal_conv(const float * x_dev, int64_t x_stride, int channels, int taps, const float * w_dev, const float * bias_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int act,
+                             float * out_dev, int64_t out_stride, void * stream);
+/* dt[t][h] = softplus(raw[t][h] + dt_bias[h]); decay[t][h] = exp(-exp(a_log[h]) * dt[t][h]); outputs [n_tok][heads] */
+PI_API int pi_op_ssd_steps(const float * raw_dev, int64_t raw_stride, const float * dt_bias_dev, const float * a_log_dev, int heads, int n_tok, float * dt_out_dev, float * decay_out_dev, void * stream);
+/* u = y * silu(z); out = u / rms(u over each of `groups` equal parts) * w */
+PI_API int pi_op_gate_group_norm(const float * y_dev, int64_t y_stride, const float * z_dev, int64_t z_stride, const float * w_dev, float eps, int n, int groups, int n_tok, float * out_dev, int64_t out_stride, void * stream);
+/* router with sigmoid scores and a choice limited to groups: the outputs form n_groups equal groups of neighbours, a group's score is the sum of its two largest scores, only outputs of the
+ * `keep` best groups can be chosen; the `top` largest scores among them win and are the weights (not renormalised) */
+PI_API int pi_op_moe_route_groups(const pi_weight * router, const float * x_dev, int64_t x_stride, int n_tok, int top, int n_groups, int keep, int exact, int32_t * sel_dev, float * selw_dev, void * stream);
+/* the grouped path with the expert's activation as a parameter (glu as for pi_op_moe_experts_act; up_dev is then [n_tok * top][2 * ff]) */
+PI_API int pi_op_moe_experts_grouped_act(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, int glu, const float * x_dev, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
+                                         float * up_dev, float * dn_dev, int32_t * idx_dev, float * out_dev, int64_t out_stride, void * stream);
+/* pi_op_moe_experts with the expert's activation as a parameter: glu = 0: relu(W_up x)^2; glu = 1: w_up holds [gate (ff rows) | up (ff rows)] per expert and the hidden values are silu(gate) * up */
+PI_API int pi_op_moe_experts_act(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, int glu, const float * x_dev, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
+                                 int exact, float * up_dev, float * out_dev, int64_t out_stride, void * stream);
 
 #ifdef __cplusplus
 }

@@ -40,7 +40,7 @@ llama_context::~llama_context() {
     if (hop_host) (void) hipHostFree(hop_host);
     pi_free(hop_dev);
     pi_free(abort_dev);
-    void * bufs[] = { lat_cache, rec_state, rec_dev, h_in, h_att, h_out, moe_w, moe_up, moe_dn, lat_scratch, rec_scratch, moe_sel, moe_idx, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
+    void * bufs[] = { cell_pos, hist, h_out2, ssd_dt, lat_cache, rec_state, rec_dev, h_in, h_att, h_out, moe_w, moe_up, moe_dn, lat_scratch, rec_scratch, moe_sel, moe_idx, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
     for (void * b : bufs) pi_free(b);
     if (rope) pi_rope_table_free(rope);
     if (stream) (void) hipStreamDestroy(stream);
@@ -49,7 +49,7 @@ llama_context::~llama_context() {
 namespace pi {
 
 static size_t kv_bytes_per_cell(const llama_context * ctx) {
-    if (ctx->model->hparams.hybrid_arch()) { size_t b = 0; for (const auto & l : ctx->model->hparams.hybrid) if (l.cache_index >= 0) b += (size_t) 4 * l.kv_rank; return b; }
+    if (ctx->model->hparams.hybrid_arch()) { size_t b = 0; for (const auto & l : ctx->model->hparams.hybrid) if (l.cache_index >= 0) b += (size_t) 4 * l.cell_floats(); return b; }
     return (size_t) 2 * 2 * ctx->model->hparams.n_embd_gqa() * (size_t) (ctx->l1 - ctx->l0);
 }
 
@@ -96,16 +96,28 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
         return false;
     }
     const int64_t t0 = time_us();
-    if (!m->ensure_loaded_hybrid(err)) return false;
+    if (pi_device_init(m->device) != 0) { err = pi_last_error(); return false; }
+    if (!m->ensure_loaded_hybrid(std::max(ctx->n_ctx, 32), err)) return false;
     ctx->t_load_us += time_us() - t0;
     if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) { err = "hipStreamCreate failed"; return false; }
     auto dev = [&](size_t bytes) -> void * { void * p = pi_malloc(std::max<size_t>(bytes, 16)); if (!p) err = pi_last_error(); return p; };
     const int nb = ctx->n_batch, width = hp.n_embd;
-    size_t lat = 0, rec = 0, in_w = 1, att_w = 1, up_w = 1, sel_w = 1, idx_n = 1;
+    size_t lat = 0, rec = 0, in_w = 1, att_w = 1, up_w = 1, sel_w = 1, idx_n = 1, step_w = 0; bool positions = false;
     ctx->lat_off.assign(hp.hybrid.size(), 0); ctx->rec_off.assign(hp.hybrid.size(), 0);
     if (hp.n_recurrent() > 0) ctx->slots.reset(new state_slots(std::max(1, ctx->n_state_slots)));
     for (size_t i = 0; i < hp.hybrid.size(); i++) {
         const pi_hybrid_layer & H = hp.hybrid[i];
+        if (H.mixer == PI_MIXER_PARALLEL) {                                  // keys | values per cell; the recurrence's matrix and the convolution's last inputs per sequence
+            const pi_gate_attention & A = H.left; const pi_ssd & R = H.right;
+            ctx->lat_off[i] = lat; lat += (size_t) ctx->n_ctx * H.cell_floats();
+            ctx->rec_off[i] = rec; rec += (size_t) ctx->slots->size() * H.state_floats();
+            ctx->rec_scratch_floats = std::max(ctx->rec_scratch_floats, pi_op_linear_attention_scratch_floats(R.heads, R.state, R.vdim, nb, ctx->slots->size()));
+            in_w = std::max(in_w, (size_t) std::max(H.in_rows(), std::max(H.mlp == PI_MLP_DENSE_RELU_SQR ? H.ff : 0, 3 * H.shared_ff)));
+            att_w = std::max(att_w, (size_t) A.heads * (A.dim + A.vdim) + (size_t) R.channels() + (size_t) R.inner());
+            step_w = std::max(step_w, (size_t) 2 * R.heads); positions = true;
+            if (H.mlp == PI_MLP_MOE_GLU) { up_w = std::max(up_w, (size_t) H.top * 2 * H.ff); sel_w = std::max(sel_w, (size_t) H.top); idx_n = std::max(idx_n, pi_op_moe_grouped_index_ints(nb, H.top, H.n_expert)); }
+            continue;
+        }
         if (H.cache_index >= 0) {
             if (ctx->n_ctx > pi_op_latent_attention_max_cells(H.kv_rank)) { err = "n_ctx = " + std::to_string(ctx->n_ctx) + " is beyond the latent-attention kernel at kv_rank " + std::to_string(H.kv_rank) + " (one score row per workgroup in LDS: n_ctx <= " + std::to_string(pi_op_latent_attention_max_cells(H.kv_rank)) + ")"; return false; }
             ctx->lat_off[i] = lat; lat += (size_t) ctx->n_ctx * H.kv_rank;
@@ -117,6 +129,8 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
     }
     if (!(ctx->rec_scratch = (float *) dev(ctx->rec_scratch_floats * 4)) || !(ctx->lat_scratch = (float *) dev(ctx->lat_scratch_floats * 4)) || !(ctx->lat_cache = (float *) dev(lat * 4)) || !(ctx->rec_state = (float *) dev(rec * 4))) return false;
     pi_memset(ctx->lat_cache, 0, std::max<size_t>(lat * 4, 16), nullptr); pi_memset(ctx->rec_state, 0, std::max<size_t>(rec * 4, 16), nullptr);
+    if (positions) { if (!(ctx->cell_pos = (int32_t *) dev((size_t) 4 * ctx->n_ctx)) || !(ctx->h_out2 = (float *) dev((size_t) 4 * nb * width)) || !(ctx->ssd_dt = (float *) dev((size_t) 4 * nb * step_w))) return false; pi_memset(ctx->cell_pos, 0, (size_t) 4 * ctx->n_ctx, nullptr); }
+    if (hp.depth_average && !(ctx->hist = (float *) dev((size_t) 4 * (hp.hybrid.size() + 1) * nb * width))) return false;
     if (!(ctx->x = (float *) dev((size_t) 4 * nb * width)) || !(ctx->nx = (float *) dev((size_t) 4 * nb * width)) || !(ctx->h_out = (float *) dev((size_t) 4 * nb * width)) ||
         !(ctx->h_in = (float *) dev((size_t) 4 * nb * in_w)) || !(ctx->h_att = (float *) dev((size_t) 4 * nb * att_w)) || !(ctx->moe_up = (float *) dev((size_t) 4 * nb * up_w)) ||
         !(ctx->moe_w = (float *) dev((size_t) 4 * nb * sel_w)) || !(ctx->moe_dn = (float *) dev((size_t) 4 * nb * sel_w * width)) || !(ctx->moe_idx = (int32_t *) dev((size_t) 4 * idx_n)) || !(ctx->moe_sel = (int32_t *) dev((size_t) 4 * nb * sel_w)) || (ctx->slots && !(ctx->rec_dev = (int32_t *) dev((size_t) 4 * nb))) ||
@@ -276,9 +290,99 @@ static bool mul_mat_grouped(int n, const pi_weight * const * ws, const void * co
 // A hybrid model's pass: per layer  x += m * N1(mixer(x)),  x += m * N2(moe(x))  — the norm sits on the sublayer's output, the sublayers read x itself; everything between the
 // matrix products is fp32.  Kernel sequence: fused input projection (activations in its epilogue) -> mixer kernel -> output projection -> norm + scale + residual; router ->
 // experts -> norm + scale + residual; final norm -> logits against the embedding table itself.
+//
+// Blocks with norms before AND after every sublayer (hp.pre_post_norm) and a learned average over depth (hp.depth_average):
+//   h = LN1(x); x += LN1b(a * attention_branch(h) + b * recurrence_branch(h));  h = LN2(x); x += LN2b(ff(h));  X_(i+1) = x;  x = sum_j c_ij X_j
+// Kernel sequence of a parallel mixer: norm -> ONE projection [q | k | v | gate | z | x | B | C | dt] -> (q/k norm + rotation, v norm, cache store) -> chunked sigmoid attention ->
+// W_o;  convolution (+ its state) -> step sizes -> recurrence -> gate + grouped norm -> W_o';  post-norm of the weighted sum + residual.  The stream after every layer is kept
+// in ctx->hist for the depth average; the block's last norm writes X_(i+1) straight into it.
+static bool forward_parallel_mixer(llama_context * ctx, const pi_hybrid_layer & H, const pi_hybrid_weights & W, size_t il, const float * N, int n_tok, int n_kv) {
+    const pi_hparams & hp = ctx->model->hparams;
+    hipStream_t s = ctx->stream;
+    const int width = hp.n_embd, ex = ctx->exact, nb = ctx->n_batch;
+    const float eps = hp.f_norm_eps;
+    const pi_gate_attention & A = H.left; const pi_ssd & R = H.right;
+    const int64_t pw = H.in_rows(), hd = (int64_t) A.heads * A.dim, hv = (int64_t) A.heads * A.vdim, gd = (int64_t) A.kv_heads * A.dim, gv = (int64_t) A.kv_heads * A.vdim;
+    float * P = ctx->h_in, * Q = ctx->h_att, * O = Q + (size_t) nb * hd, * C = O + (size_t) nb * hv, * S = C + (size_t) nb * R.channels();
+    float * kc = ctx->lat_cache + ctx->lat_off[il], * vc = kc + (size_t) ctx->n_ctx * gd;
+    float * ssm = ctx->rec_state + ctx->rec_off[il], * conv_state = ssm + (size_t) ctx->slots->size() * R.heads * R.state * R.vdim;
+    OP_OK(pi_op_dense(W.w_in, N, width, n_tok, P, pw, PI_ACT_NONE, pw, PI_ACT_NONE, ex, s));
+    // attention branch
+    OP_OK(pi_op_qkv_prepare(P, P + hd, P + hd + gd, pw, W.q_norm, W.k_norm, eps, A.heads, A.kv_heads, A.dim, A.vdim, W.rotary, ctx->pos_dev, n_tok, Q, hd, kc, vc, ctx->cell_pos, ctx->dyn_dev, s));
+    OP_OK(pi_op_chunk_attention(Q, hd, kc, vc, ctx->cell_pos, ctx->mask_dev, ctx->pos_dev, W.head_bias, P + hd + gd + gv, pw, PI_ACT_SIGMOID, A.scale, A.chunk, A.heads, A.kv_heads, A.dim, A.vdim, n_tok, n_kv, O, hv, ctx->dyn_dev, s));
+    trace(ctx, "att", (int) il, O, hv, n_tok);
+    OP_OK(pi_op_dense(W.w_o, O, hv, n_tok, ctx->h_out, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+    // recurrence branch
+    const float * R0 = P + A.in_rows();                                   // z | x B C | dt
+    const int inner = R.inner(), gn = R.groups * R.state;
+    float * dt = ctx->ssd_dt, * decay = dt + (size_t) nb * R.heads;
+    OP_OK(pi_op_causal_conv(R0 + inner, pw, R.channels(), R.conv, W.conv_w, W.conv_b, conv_state, ctx->rec_dev, n_tok, PI_ACT_SILU, C, R.channels(), s));
+    OP_OK(pi_op_ssd_steps(R0 + inner + R.channels(), pw, W.dt_bias, W.a_log, R.heads, n_tok, dt, decay, s));
+    OP_OK(pi_op_linear_attention_ex(C + inner + gn, C + inner, C, R.channels(), R.heads, R.groups, R.state, R.vdim, nullptr, decay, dt, R.heads, W.skip, ssm, ctx->rec_dev, n_tok, ctx->slots->size(),
+                                    ctx->rec_scratch, ctx->rec_scratch_floats, S, inner, s));
+    OP_OK(pi_op_gate_group_norm(S, inner, R0, pw, W.mix_norm, eps, inner, R.norm_groups, n_tok, S, inner, s));
+    trace(ctx, "ssd", (int) il, S, inner, n_tok);
+    OP_OK(pi_op_dense(W.w_o2, S, inner, n_tok, ctx->h_out2, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+    return true;
+}
+
+static bool forward_pre_post_blocks(llama_context * ctx, int n_tok, int n_kv) {
+    llama_model * m = ctx->model;
+    const pi_hparams & hp = m->hparams;
+    hipStream_t s = ctx->stream;
+    const int width = hp.n_embd, ex = ctx->exact, nb = ctx->n_batch;
+    const float eps = hp.f_norm_eps;
+    const size_t hs = (size_t) nb * width;
+    float * P = ctx->h_in, * N = ctx->nx, * Y = ctx->h_out, * Y2 = ctx->h_out2;
+    float * x = hp.depth_average ? ctx->hist : ctx->x;                    // the embedding output is X_0
+    OP_OK(pi_op_embed(m->tok_embd, ctx->tokens_dev, n_tok, hp.embed_scale, x, s));
+    for (size_t il = 0; il < hp.hybrid.size(); il++) {
+        const pi_hybrid_layer & H = hp.hybrid[il];
+        const pi_hybrid_weights & W = m->hweights[(size_t) H.weights];
+        float * X_next = hp.depth_average ? ctx->hist + (il + 1) * hs : ctx->x;     // where the block's result goes
+        float * after_mixer = H.has_mlp ? ctx->x : X_next;
+        OP_OK(pi_op_layer_norm_mix(x, width, 1.0f, nullptr, 0, 0.0f, W.norm1, W.norm1_b, eps, width, n_tok, nullptr, 0, N, width, s));
+        if (H.mixer != PI_MIXER_PARALLEL) { ctx->last_error = "blocks with norms on both sides of a sublayer are built for the parallel mixer"; return false; }
+        if (!forward_parallel_mixer(ctx, H, W, il, N, n_tok, n_kv)) return false;
+        OP_OK(pi_op_layer_norm_mix(Y, width, H.left_scale, Y2, width, H.right_scale, W.post1, W.post1_b, eps, width, n_tok, x, width, after_mixer, width, s));
+        if (H.has_mlp) {
+            x = after_mixer;
+            OP_OK(pi_op_layer_norm_mix(x, width, 1.0f, nullptr, 0, 0.0f, W.norm2, W.norm2_b, eps, width, n_tok, nullptr, 0, N, width, s));
+            if (H.mlp == PI_MLP_DENSE_RELU_SQR) {
+                OP_OK(pi_op_dense(W.ff_up, N, width, n_tok, P, H.ff, PI_ACT_RELU_SQR, H.ff, PI_ACT_RELU_SQR, ex, s));
+                OP_OK(pi_op_dense(W.ff_down, P, H.ff, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+                OP_OK(pi_op_layer_norm_mix(Y, width, 1.0f, nullptr, 0, 0.0f, W.post2, W.post2_b, eps, width, n_tok, x, width, X_next, width, s));
+            } else {
+                OP_OK(pi_op_moe_route_groups(W.router, N, width, n_tok, H.top, H.route_groups, H.route_keep, ex, ctx->moe_sel, ctx->moe_w, s));
+                if (pi_op_moe_grouped_ok(W.e_up, W.e_down, H.n_expert, H.ff, 1, n_tok, H.top, ex))                                                // prompts: by expert, on the matrix cores
+                    OP_OK(pi_op_moe_experts_grouped_act(W.e_up, W.e_down, H.n_expert, H.ff, 1, N, width, ctx->moe_sel, ctx->moe_w, n_tok, H.top, ctx->moe_up, ctx->moe_dn, ctx->moe_idx, Y, width, s));
+                else
+                    OP_OK(pi_op_moe_experts_act(W.e_up, W.e_down, H.n_expert, H.ff, 1, N, width, ctx->moe_sel, ctx->moe_w, n_tok, H.top, ex, ctx->moe_up, Y, width, s));
+                if (H.shared_ff > 0) {                                     // the expert every token uses: silu(gate) in the projection's epilogue, * up, down
+                    const int sf = H.shared_ff;
+                    float * G = P + (size_t) nb * 2 * sf;
+                    OP_OK(pi_op_dense(W.ff_up, N, width, n_tok, P, 2 * sf, PI_ACT_SILU, sf, PI_ACT_NONE, ex, s));
+                    OP_OK(pi_op_glu_mul(P, 2 * sf, sf, n_tok, G, sf, s));
+                    OP_OK(pi_op_dense(W.ff_down, G, sf, n_tok, Y2, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+                }
+                OP_OK(pi_op_layer_norm_mix(Y, width, 1.0f, H.shared_ff > 0 ? Y2 : nullptr, width, 1.0f, W.post2, W.post2_b, eps, width, n_tok, x, width, X_next, width, s));
+            }
+        }
+        x = X_next;
+        if (hp.depth_average) { OP_OK(pi_op_depth_mix(ctx->hist, (int64_t) hs, (int) il + 2, W.depth, width, n_tok, ctx->x, width, s)); x = ctx->x; }
+        trace(ctx, "lout", (int) il, x, width, n_tok);
+    }
+    OP_OK(pi_op_layer_norm_mix(x, width, 1.0f, nullptr, 0, 0.0f, m->output_norm, m->output_norm_b, eps, width, n_tok, nullptr, 0, N, width, s));
+    OP_OK(pi_op_dense(hp.own_head ? m->output : m->tok_embd, N, width, n_tok, ctx->logits_dev, hp.n_vocab, PI_ACT_NONE, hp.n_vocab, PI_ACT_NONE, ex, s));
+    if (hp.logit_softcap > 0.0f) OP_OK(pi_op_softcap(ctx->logits_dev, (int64_t) n_tok * hp.n_vocab, hp.logit_softcap, s));
+    OP_OK(pi_op_topk(ctx->logits_dev, hp.n_vocab, n_tok, 8, ctx->topk_ids_dev, ctx->topk_vals_dev, ctx->topk_sum_dev, ctx->topk_scratch_dev, s));
+    return true;
+}
+
 static bool forward_hybrid(llama_context * ctx, int n_tok, int n_kv) {
     llama_model * m = ctx->model;
     const pi_hparams & hp = m->hparams;
+    if (hp.pre_post_norm) return forward_pre_post_blocks(ctx, n_tok, n_kv);
     hipStream_t s = ctx->stream;
     const int width = hp.n_embd, ex = ctx->exact;
     const float eps = hp.f_norm_rms_eps, rm = hp.residual_mult;
@@ -304,7 +408,7 @@ static bool forward_hybrid(llama_context * ctx, int n_tok, int n_kv) {
         OP_OK(pi_op_rms_scale(Y, width, W.norm1, 1.0f, eps, width, n_tok, nullptr, 0, x, width, rm, x, width, nullptr, 0, s));
         if (H.has_mlp) {
             OP_OK(pi_op_moe_route(W.router, W.correction, x, width, n_tok, H.top, ex, ctx->moe_sel, ctx->moe_w, s));
-            if (pi_op_moe_grouped_ok(W.e_up, W.e_down, H.n_expert, H.ff, n_tok, H.top, ex))                                                        // prompts: by expert, on the matrix cores
+            if (pi_op_moe_grouped_ok(W.e_up, W.e_down, H.n_expert, H.ff, 0, n_tok, H.top, ex))                                                     // prompts: by expert, on the matrix cores
                 OP_OK(pi_op_moe_experts_grouped(W.e_up, W.e_down, H.n_expert, H.ff, x, width, ctx->moe_sel, ctx->moe_w, n_tok, H.top, ctx->moe_up, ctx->moe_dn, ctx->moe_idx, Y, width, s));
             else
                 OP_OK(pi_op_moe_experts(W.e_up, W.e_down, H.n_expert, H.ff, x, width, ctx->moe_sel, ctx->moe_w, n_tok, H.top, ex, ctx->moe_up, Y, width, s));

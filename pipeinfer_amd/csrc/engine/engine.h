@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <condition_variable>
 #include <mutex>
@@ -31,7 +32,8 @@
 
 // LLAMA and FALCON have their own blocks in forward(); the others are one generic sequential block (norm -> attention -> + -> norm -> MLP -> +) described by pi_block below
 enum pi_arch { PI_ARCH_LLAMA = 0, PI_ARCH_FALCON = 1, PI_ARCH_BAICHUAN = 2, PI_ARCH_STARCODER = 3, PI_ARCH_REFACT = 4, PI_ARCH_BLOOM = 5, PI_ARCH_MPT = 6, PI_ARCH_STABLELM = 7, PI_ARCH_PERSIMMON = 8,
-               PI_ARCH_FASOVIK = 9 /* a hybrid model: a list of layers, each with its own mixer (pi_hybrid_layer), read from config.json + model.safetensors */ };
+               PI_ARCH_FASOVIK = 9 /* a hybrid model: a list of layers, each with its own mixer (pi_hybrid_layer), read from config.json + model.safetensors */,
+               PI_ARCH_VIKARAX = 10 /* hybrid as well: layer norms before and after every sublayer, a learned average over depth, mixers of two parallel branches */ };
 
 // what the reference's build_* functions differ in (llama.cpp:3985-4104 baichuan, 4229-4327 starcoder, 4540-4630 refact, 4632-4725 bloom, 4727-4825 mpt, 4827-4939 stablelm)
 struct pi_block {
@@ -48,21 +50,41 @@ struct pi_block {
 // One layer of a hybrid model.  The mixer is one of the mechanisms below, each with its sizes and constants as the model's description gives them; the feed-forward is a
 // mixture of experts (or absent).  A layer may use another layer's tensors (`weights`) while keeping a cache / state of its own.
 enum pi_mixer_kind { PI_MIXER_LATENT_ATTENTION = 0,   // keys / values are up-projections of one cached low-rank latent, no positions, causal, soft-max with a per-head sink
-                     PI_MIXER_LIGHTNING = 1 };        // linear attention with a per-head decay: a [dim][vdim] state per head and sequence
+                     PI_MIXER_LIGHTNING = 1,          // linear attention with a per-head decay: a [dim][vdim] state per head and sequence
+                     PI_MIXER_PARALLEL = 2 };         // two branches that read the same input, summed with fixed factors: chunked sigmoid attention (pi_gate_attention) + a selective recurrence (pi_ssd)
+// attention with grouped key / value heads, normed and partly rotated q / k, unit-norm values, un-normalised sigmoid weights inside chunks of positions, a per-head output gate
+struct pi_gate_attention { int heads = 0, kv_heads = 0, dim = 0, vdim = 0, rot_dims = 0, chunk = 0; float rot_base = 10000.0f, scale = 1.0f;
+                           int in_rows() const { return heads * dim + kv_heads * (dim + vdim) + heads; } };                      // [q | k | v | gate]
+// selective state-space recurrence: a [state][vdim] matrix per head and sequence, B / C shared by the heads of a group, a causal convolution of `conv` taps over x, B, C
+struct pi_ssd { int heads = 0, vdim = 0, state = 0, groups = 0, conv = 0, norm_groups = 1;
+                int inner() const { return heads * vdim; } int channels() const { return inner() + 2 * groups * state; } int in_rows() const { return 2 * inner() + 2 * groups * state + heads; }   // [z | x | B | C | dt]
+                size_t state_floats() const { return (size_t) heads * state * vdim + (size_t) std::max(conv - 1, 0) * channels(); } };
+enum pi_mlp_kind { PI_MLP_NONE = 0, PI_MLP_MOE_RELU_SQR = 1 /* routed by a soft-max with correction, experts relu(up)^2, identity experts */, PI_MLP_DENSE_RELU_SQR = 2,
+                   PI_MLP_MOE_GLU = 3 /* routed by sigmoid scores inside the best groups, experts silu(gate) * up, an optional shared expert */ };
 struct pi_hybrid_layer {
     pi_mixer_kind mixer = PI_MIXER_LATENT_ATTENTION;
     int weights = 0;                                  // index of the layer that owns the tensors (its own index unless shared)
     int heads = 0, dim = 0, vdim = 0, kv_rank = 0;
     float scale = 1.0f;                               // latent attention: factor on q . k
     std::vector<float> decay;                         // lightning: per head
+    pi_gate_attention left; pi_ssd right; float left_scale = 1.0f, right_scale = 1.0f;      // PI_MIXER_PARALLEL
     bool has_mlp = false; int n_expert = 0, n_identity = 0, top = 0, ff = 0;
-    int cache_index = -1, state_index = -1;           // ordinal among the layers that keep a latent cache / a recurrent state
-    int in_rows() const { return mixer == PI_MIXER_LIGHTNING ? 2 * heads * dim + 2 * heads * vdim : heads * dim + kv_rank; }     // rows of the fused input projection
+    pi_mlp_kind mlp = PI_MLP_NONE; int route_groups = 0, route_keep = 0, shared_ff = 0;     // (has_mlp <=> mlp != PI_MLP_NONE)
+    int cache_index = -1, state_index = -1;           // ordinal among the layers that keep a per-cell cache / a recurrent state
+    int in_rows() const { return mixer == PI_MIXER_PARALLEL ? left.in_rows() + right.in_rows() : mixer == PI_MIXER_LIGHTNING ? 2 * heads * dim + 2 * heads * vdim : heads * dim + kv_rank; }     // rows of the fused input projection
+    int out_cols() const { return mixer == PI_MIXER_PARALLEL ? std::max(left.heads * left.vdim, right.inner()) : heads * vdim; }                                                   // widest input of an output projection
+    size_t cell_floats() const { return mixer == PI_MIXER_PARALLEL ? (size_t) left.kv_heads * (left.dim + left.vdim) : mixer == PI_MIXER_LATENT_ATTENTION ? (size_t) kv_rank : 0; }   // cached per cell
+    size_t state_floats() const { return mixer == PI_MIXER_PARALLEL ? right.state_floats() : mixer == PI_MIXER_LIGHTNING ? (size_t) heads * dim * vdim : 0; }                       // kept per sequence
 };
 struct pi_hybrid_weights {                            // the tensors of a layer that owns some
     pi_weight * w_in = nullptr;                       // latent attention: [q | dkv], lightning: [q | k | v | g] (projections of the same input, one matrix)
     pi_weight * w_uk = nullptr, * w_uv = nullptr, * w_o = nullptr, * router = nullptr, * e_up = nullptr, * e_down = nullptr;
     float * norm1 = nullptr, * norm2 = nullptr, * mix_norm = nullptr, * sink = nullptr, * decay = nullptr, * correction = nullptr;
+    // parallel mixer: w_in = [q | k | v | gate | z | x | B | C | dt], w_o = the attention branch's output projection, w_o2 = the recurrence's; dense / shared feed-forward: [up] or [gate | up], down
+    pi_weight * w_o2 = nullptr, * ff_up = nullptr, * ff_down = nullptr;
+    float * norm1_b = nullptr, * norm2_b = nullptr, * post1 = nullptr, * post1_b = nullptr, * post2 = nullptr, * post2_b = nullptr, * depth = nullptr;      // biases of the pre-norms, the post-norms, the depth average's factors
+    float * q_norm = nullptr, * k_norm = nullptr, * head_bias = nullptr, * conv_w = nullptr, * conv_b = nullptr, * dt_bias = nullptr, * a_log = nullptr, * skip = nullptr;
+    void * rotary = nullptr;                          // pi_rotary_table of the layer's (dims, base)
     bool loaded = false;
 };
 
@@ -74,12 +96,15 @@ struct pi_hparams {
     pi_block block;
     std::vector<pi_hybrid_layer> hybrid;          // PI_ARCH_FASOVIK: the layers in order
     float embed_scale = 1.0f, residual_mult = 1.0f;
-    bool hybrid_arch() const { return arch == PI_ARCH_FASOVIK; }
+    // what the hybrid architectures' blocks differ in: layer norms (weight, bias) before AND after every sublayer or an RMS norm (1 + w) on its output only; the stream that
+    // goes on after a layer = a learned weighted sum of the embedding output and every layer's result so far; an output head of its own or the embedding table; tanh cap on the logits
+    bool pre_post_norm = false, depth_average = false, own_head = false; float logit_softcap = 0.0f;
+    bool hybrid_arch() const { return arch == PI_ARCH_FASOVIK || arch == PI_ARCH_VIKARAX; }
     int n_latent() const { int n = 0; for (const auto & l : hybrid) n += l.cache_index >= 0; return n; }
     int n_recurrent() const { int n = 0; for (const auto & l : hybrid) n += l.state_index >= 0; return n; }
     int head_dim() const { return n_embd / n_head; }
     int n_embd_gqa() const { return head_dim() * n_head_kv; }
-    bool generic() const { return arch != PI_ARCH_LLAMA && arch != PI_ARCH_FALCON && arch != PI_ARCH_FASOVIK; }
+    bool generic() const { return arch != PI_ARCH_LLAMA && arch != PI_ARCH_FALCON && !hybrid_arch(); }
 };
 
 struct pi_layer {
@@ -106,6 +131,7 @@ struct llama_model {
     float * alibi_slopes = nullptr;                                                              // f32 [n_head] on the device when block.alibi > 0
     std::vector<pi_layer> layers;
     std::vector<void *> f32_allocs;
+    std::vector<void *> retired_tables;       // rotation tables a context with a longer n_ctx replaced (earlier contexts may still read them)
     struct matrix_ref { pi_weight * w; const void * host; int layer; };                           // every uploaded matrix with its GGUF bytes (layer -1: embeddings / output head)
     std::vector<matrix_ref> matrices;
     bool output_has_mq = false;
@@ -116,7 +142,7 @@ struct llama_model {
     // uploads (once) token_embd if first, layers [l0,l1), final norm + output if last
     // want_mq: also make the tile-major copies of the K-quant matrices (contexts whose widest pass reaches the matrix-core kernel)
     bool ensure_loaded(int l0, int l1, bool first, bool last, bool want_mq, std::string & err);
-    bool ensure_loaded_hybrid(std::string & err);
+    bool ensure_loaded_hybrid(int n_positions, std::string & err);      // n_positions: the context length the rotation tables must cover
     size_t stage_weight_bytes(int l0, int l1, bool first, bool last, int n_tok) const;
 };
 
@@ -185,6 +211,8 @@ struct llama_context {
     // hybrid models: latent cache [cells][kv_rank] fp32 per latent-attention layer (cells = the kv_cells table above), recurrent states [slots][heads][dim][vdim] fp32 per
     // lightning layer (slots = state_slots), both at per-layer offsets into one allocation each
     float * lat_cache = nullptr, * rec_state = nullptr; std::vector<size_t> lat_off, rec_off;
+    int32_t * cell_pos = nullptr;                             // position of every cell's token, on the device (mixers that look at positions besides the mask: chunks)
+    float * hist = nullptr, * h_out2 = nullptr, * ssd_dt = nullptr;   // depth average: the stream after the embedding and after every layer [n_layer + 1][n_batch][width]; second branch output; step sizes | decays
     std::unique_ptr<pi::state_slots> slots; int n_state_slots = 8;
     int32_t * rec_dev = nullptr;                              // per token of the pass: state slot (| 1 << 30: start from zero)
     int exact = 0;                                            // 1: dense operators keep fp32 activations (pipeinfer_context_set_precision)

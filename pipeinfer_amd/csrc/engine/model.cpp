@@ -39,7 +39,9 @@ llama_model::~llama_model() {
         pi_weight_free(l.wq); pi_weight_free(l.wk); pi_weight_free(l.wv); pi_weight_free(l.wo); pi_weight_free(l.wqkv);
         pi_weight_free(l.ffn_gate); pi_weight_free(l.ffn_down); pi_weight_free(l.ffn_up);
     }
-    for (auto & w : hweights) { pi_weight_free(w.w_in); pi_weight_free(w.w_uk); pi_weight_free(w.w_uv); pi_weight_free(w.w_o); pi_weight_free(w.router); pi_weight_free(w.e_up); pi_weight_free(w.e_down); }
+    for (auto & w : hweights) { pi_weight_free(w.w_in); pi_weight_free(w.w_uk); pi_weight_free(w.w_uv); pi_weight_free(w.w_o); pi_weight_free(w.router); pi_weight_free(w.e_up); pi_weight_free(w.e_down);
+                                pi_weight_free(w.w_o2); pi_weight_free(w.ff_up); pi_weight_free(w.ff_down); if (w.rotary) pi_rotary_table_free(w.rotary); }
+    for (void * t : retired_tables) pi_rotary_table_free(t);
     pi_weight_free(tok_embd); pi_weight_free(output); pi_weight_free(pos_embd);
     for (void * p : f32_allocs) pi_free(p);
 }
@@ -186,11 +188,17 @@ size_t llama_model::stage_weight_bytes(int l0, int l1, bool first, bool last, in
         for (size_t i = 0; i < hparams.hybrid.size(); i++) {
             const pi_hybrid_layer & H = hparams.hybrid[i];
             const size_t w = (size_t) hparams.n_embd;
+            if (H.mixer == PI_MIXER_PARALLEL) {                                // both branches' projections, the norms' vectors, the feed-forward a token uses
+                b += 2 * (size_t) H.in_rows() * w + 2 * ((size_t) H.left.heads * H.left.vdim + H.right.inner()) * w + 4 * 8 * w;
+                if (H.mlp == PI_MLP_DENSE_RELU_SQR) b += 4 * (size_t) H.ff * w;
+                if (H.mlp == PI_MLP_MOE_GLU) b += 2 * (size_t) H.n_expert * w + (size_t) std::min(H.n_expert, std::max(1, n_tok) * H.top) * 6 * (size_t) H.ff * w + 6 * (size_t) H.shared_ff * w;
+                continue;
+            }
             b += 2 * (size_t) H.in_rows() * w + 2 * (size_t) H.heads * H.vdim * w + 4 * w;
             if (H.mixer == PI_MIXER_LATENT_ATTENTION) b += 2 * (size_t) H.kv_rank * H.heads * (H.dim + H.vdim);
             if (H.has_mlp) b += 2 * (size_t) (H.n_expert + H.n_identity) * w + (size_t) std::min(H.n_expert, std::max(1, n_tok) * H.top) * 4 * (size_t) H.ff * w;
         }
-        return b + 2 * (size_t) hparams.n_vocab * hparams.n_embd + 2 * (size_t) n_tok * hparams.n_embd;
+        return b + 2 * (size_t) hparams.n_vocab * hparams.n_embd + 2 * (size_t) n_tok * hparams.n_embd;      // (the output matrix once — the embedding table itself or a head of its own — + the tokens' embedding rows)
     }
     auto add = [&](const std::string & name, int64_t rows_used) {
         const pi::gguf_tensor * t = file.tensor(name);

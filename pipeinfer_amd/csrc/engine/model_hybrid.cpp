@@ -4,6 +4,11 @@
 // kv_rank + scale | decay[] }, mlp: null | { kind: "moe", expert.ff, router.experts / identity / top }, weights_of: j (optional: the layer has no tensors, it uses layer j's) }.
 // Tensors: embed, final.norm, l<i>.norm1 / norm2, l<i>.mix.{q, dkv, dkv.norm, uk, uv, sink, o} or l<i>.mix.{q, k, v, g, o, norm}, l<i>.mlp.{router, correction, e<k>.up, e<k>.down}.
 // Projections that read the same input are uploaded as ONE matrix (rows one after the other) so that they are one launch; vectors go up as fp32.
+//
+// Vikarax (same files, other keys): vocab, width, norm.eps, logit_softcap, layers[]: { type: "parallel", mixer: { left: { heads, kv_heads, dim, vdim, scale, rot.dims / rot.base,
+// mask.size }, right: { heads, vdim, state, groups, conv, norm_groups }, left_scale, right_scale }, mlp: null | { kind: "dense", ff } | { kind: "moe", expert.ff, router.experts /
+// top / groups.count / groups.keep, shared.ff } }.  Tensors: embed, head, final.norm (+ .b), l<i>.norm1 / norm1b / norm2 / norm2b (+ .b), l<i>.dwa, l<i>.mix.left.{q, k, v, q.norm,
+// k.norm, pb, g, o}, l<i>.mix.right.{in, conv, conv.b, dt_bias, A_log, D, norm, o}, l<i>.mlp.{up, down} or l<i>.mlp.{router, e<k>.{gate, up, down}, shared.{gate, up, down}}.
 #include "engine.h"
 #include "json.h"
 
@@ -58,6 +63,13 @@ struct loader {
         m.f32_allocs.push_back(d); m.hbm_bytes += v.size() * 4;
         return d;
     }
+    float * vector2(const std::string & name, int64_t rows, int64_t cols) {      // a small [rows][cols] table widened to fp32, as stored
+        const pi::st_tensor * t = get(name, { rows, cols });
+        if (!t) return nullptr;
+        std::vector<float> v((size_t) (rows * cols));
+        for (size_t i = 0; i < v.size(); i++) v[i] = bf16_to_f32(((const uint16_t *) t->data)[i]);
+        return vector_f32(v);
+    }
     float * vector(const std::string & name, int64_t n) {
         const pi::st_tensor * t = get(name, { n });
         if (!t) return nullptr;
@@ -67,9 +79,74 @@ struct loader {
     }
 };
 
+
+// Vikarax: every layer is a parallel mixer (attention branch + recurrence) with an optional dense or routed feed-forward
+static bool read_vikarax_config(const pi::json & cfg, pi_hparams & hp, std::string & what) {
+    using pi::json;
+    double d;
+    if (!num_at(cfg, "norm.eps", d)) { what = "no 'norm.eps'"; return false; }
+    hp.f_norm_eps = hp.f_norm_rms_eps = (float) d;
+    hp.logit_softcap = num_at(cfg, "logit_softcap", d) ? (float) d : 0.0f;
+    hp.pre_post_norm = hp.depth_average = hp.own_head = true;
+    const json * layers = cfg.find("layers");
+    if (!layers || !layers->is_arr() || layers->arr.empty()) { what = "'layers' must be a non-empty list"; return false; }
+    hp.n_layer = (int) layers->arr.size();
+    hp.n_head = hp.n_head_kv = 1; hp.n_ctx_train = 0;
+    int n_cache = 0, n_state = 0;
+    for (int i = 0; i < hp.n_layer; i++) {
+        const json & jl = layers->arr[(size_t) i];
+        const std::string where = "layers[" + std::to_string(i) + "]: ";
+        auto bad = [&](const std::string & w) { what = where + w; return false; };
+        pi_hybrid_layer H;
+        const json * type = jl.find("type");
+        if (!type || !type->is_str() || type->str != "parallel") return bad("mixer type must be 'parallel'");
+        H.mixer = PI_MIXER_PARALLEL; H.weights = i;
+        pi_gate_attention & A = H.left; pi_ssd & R = H.right;
+        if (!int_at(jl, "mixer.left.heads", A.heads) || !int_at(jl, "mixer.left.kv_heads", A.kv_heads) || !int_at(jl, "mixer.left.dim", A.dim) || !int_at(jl, "mixer.left.vdim", A.vdim) ||
+            A.heads < 1 || A.kv_heads < 1 || A.heads % A.kv_heads || A.dim < 1 || A.vdim < 1) return bad("mixer.left needs positive 'heads', 'kv_heads' (a divisor of heads), 'dim', 'vdim'");
+        if (!num_at(jl, "mixer.left.scale", d)) return bad("mixer.left needs 'scale'");
+        A.scale = (float) d;
+        if (jl.at("mixer.left.rot") && !jl.at("mixer.left.rot")->is_null()) {
+            if (!int_at(jl, "mixer.left.rot.dims", A.rot_dims) || !num_at(jl, "mixer.left.rot.base", d) || (A.rot_dims & 1) || A.rot_dims > A.dim) return bad("mixer.left.rot needs an even 'dims' <= dim and 'base'");
+            A.rot_base = (float) d;
+        }
+        if (jl.at("mixer.left.mask") && !jl.at("mixer.left.mask")->is_null() && (!int_at(jl, "mixer.left.mask.size", A.chunk) || A.chunk < 1)) return bad("mixer.left.mask needs a positive 'size'");
+        if (!int_at(jl, "mixer.right.heads", R.heads) || !int_at(jl, "mixer.right.vdim", R.vdim) || !int_at(jl, "mixer.right.state", R.state) || !int_at(jl, "mixer.right.groups", R.groups) ||
+            !int_at(jl, "mixer.right.conv", R.conv) || R.heads < 1 || R.vdim < 1 || R.state < 1 || R.groups < 1 || R.heads % R.groups || R.conv < 1 || R.conv > 64)
+            return bad("mixer.right needs positive 'heads', 'vdim', 'state', 'groups' (a divisor of heads) and 'conv' (1..64)");
+        if (R.state > 1024) return bad("mixer.right.state above 1024");
+        R.norm_groups = 1;
+        if (jl.at("mixer.right.norm_groups") && (!int_at(jl, "mixer.right.norm_groups", R.norm_groups) || R.norm_groups < 1 || R.inner() % R.norm_groups)) return bad("mixer.right.norm_groups must divide heads * vdim");
+        if (!num_at(jl, "mixer.left_scale", d)) return bad("mixer needs 'left_scale'");
+        H.left_scale = (float) d;
+        if (!num_at(jl, "mixer.right_scale", d)) return bad("mixer needs 'right_scale'");
+        H.right_scale = (float) d;
+        H.heads = A.heads; H.dim = A.dim; H.vdim = A.vdim;
+        H.cache_index = n_cache++; H.state_index = n_state++;
+        if (jl.has("mlp")) {
+            const json * kind = jl.at("mlp.kind");
+            if (!kind || !kind->is_str()) return bad("mlp needs 'kind'");
+            if (kind->str == "dense") {
+                if (!int_at(jl, "mlp.ff", H.ff) || H.ff < 1) return bad("a dense mlp needs 'ff'");
+                H.mlp = PI_MLP_DENSE_RELU_SQR;
+            } else if (kind->str == "moe") {
+                if (!int_at(jl, "mlp.router.experts", H.n_expert) || !int_at(jl, "mlp.router.top", H.top) || !int_at(jl, "mlp.expert.ff", H.ff) || H.n_expert < 1 || H.ff < 1 || H.top < 1) return bad("a routed mlp needs 'router.experts', 'router.top', 'expert.ff'");
+                H.route_groups = H.route_keep = 1;
+                if (jl.at("mlp.router.groups") && !jl.at("mlp.router.groups")->is_null() && (!int_at(jl, "mlp.router.groups.count", H.route_groups) || !int_at(jl, "mlp.router.groups.keep", H.route_keep))) return bad("mlp.router.groups needs 'count' and 'keep'");
+                if (H.route_groups < 1 || H.n_expert % H.route_groups || H.route_keep < 1 || H.route_keep > H.route_groups || H.top > H.route_keep * (H.n_expert / H.route_groups)) return bad("the router's groups must divide the experts, and the kept groups must hold at least 'top' experts");
+                if (jl.at("mlp.shared") && !jl.at("mlp.shared")->is_null() && (!int_at(jl, "mlp.shared.ff", H.shared_ff) || H.shared_ff < 1)) return bad("mlp.shared needs 'ff'");
+                H.mlp = PI_MLP_MOE_GLU;
+            } else return bad("feed-forward kind '" + kind->str + "' is unknown (dense, moe)");
+            H.has_mlp = true;
+        }
+        hp.hybrid.push_back(std::move(H));
+    }
+    return true;
+}
+
 }  // namespace
 
-bool llama_model::ensure_loaded_hybrid(std::string & err) {
+bool llama_model::ensure_loaded_hybrid(int n_positions, std::string & err) {
     const pi_hparams & hp = hparams;
     loader L{ *this, err };
     pi_weight_set_mq_copies(0);
@@ -79,11 +156,48 @@ bool llama_model::ensure_loaded_hybrid(std::string & err) {
         if (!(tok_embd = L.matrix({ { "embed", hp.n_vocab } }, width))) return false;
         if (!(output_norm = L.vector("final.norm", width))) return false;
     }
+    if (hp.own_head && !output) {
+        if (!(output = L.matrix({ { "head", hp.n_vocab } }, width))) return false;
+        if (!(output_norm_b = L.vector("final.norm.b", width))) return false;
+    }
     for (size_t i = 0; i < hp.hybrid.size(); i++) {
         const pi_hybrid_layer & H = hp.hybrid[i];
         pi_hybrid_weights & W = hweights[i];
+        if (H.weights == (int) i && W.loaded && W.rotary && pi_rotary_table_positions(W.rotary) < n_positions) {        // a later context is longer than the table
+            void * t = pi_rotary_table_create(n_positions, H.left.rot_dims, H.left.rot_base);
+            if (!t) { err = std::string("rotation table: ") + pi_last_error(); return false; }
+            retired_tables.push_back(W.rotary); W.rotary = t;
+        }
         if (H.weights != (int) i || W.loaded) continue;
         const std::string p = "l" + std::to_string(i) + ".";
+        if (H.mixer == PI_MIXER_PARALLEL) {
+            const pi_gate_attention & A = H.left; const pi_ssd & R = H.right;
+            const std::string l = p + "mix.left.", r = p + "mix.right.";
+            struct { float ** w, ** b; const char * name; bool need; } norms[] = { { &W.norm1, &W.norm1_b, "norm1", true }, { &W.post1, &W.post1_b, "norm1b", true },
+                                                                                   { &W.norm2, &W.norm2_b, "norm2", H.has_mlp }, { &W.post2, &W.post2_b, "norm2b", H.has_mlp } };
+            for (auto & n : norms) if (n.need && (!(*n.w = L.vector(p + n.name, width)) || !(*n.b = L.vector(p + n.name + ".b", width)))) return false;
+            if (hp.depth_average && !(W.depth = L.vector(p + "dwa", (int64_t) i + 2))) return false;
+            if (!(W.w_in = L.matrix({ { l + "q", (int64_t) A.heads * A.dim }, { l + "k", (int64_t) A.kv_heads * A.dim }, { l + "v", (int64_t) A.kv_heads * A.vdim }, { l + "g", A.heads }, { r + "in", R.in_rows() } }, width))) return false;
+            if (!(W.q_norm = L.vector(l + "q.norm", A.dim)) || !(W.k_norm = L.vector(l + "k.norm", A.dim)) || !(W.head_bias = L.vector(l + "pb", A.heads))) return false;
+            if (!(W.w_o = L.matrix({ { l + "o", width } }, (int64_t) A.heads * A.vdim)) || !(W.w_o2 = L.matrix({ { r + "o", width } }, R.inner()))) return false;
+            if (!(W.conv_w = L.vector2(r + "conv", R.channels(), R.conv)) || !(W.conv_b = L.vector(r + "conv.b", R.channels()))) return false;
+            if (!(W.dt_bias = L.vector(r + "dt_bias", R.heads)) || !(W.a_log = L.vector(r + "A_log", R.heads)) || !(W.skip = L.vector(r + "D", R.heads)) || !(W.mix_norm = L.vector(r + "norm", R.inner()))) return false;
+            if (!(W.rotary = pi_rotary_table_create(std::max(n_positions, 32), A.rot_dims, A.rot_base))) { err = std::string("rotation table: ") + pi_last_error(); return false; }
+            if (H.mlp == PI_MLP_DENSE_RELU_SQR) {
+                if (!(W.ff_up = L.matrix({ { p + "mlp.up", H.ff } }, width)) || !(W.ff_down = L.matrix({ { p + "mlp.down", width } }, H.ff))) return false;
+            } else if (H.mlp == PI_MLP_MOE_GLU) {
+                if (!(W.router = L.matrix({ { p + "mlp.router", H.n_expert } }, width))) return false;
+                std::vector<std::pair<std::string, int64_t>> ups, downs;
+                for (int e = 0; e < H.n_expert; e++) {
+                    const std::string q = p + "mlp.e" + std::to_string(e) + ".";
+                    ups.push_back({ q + "gate", H.ff }); ups.push_back({ q + "up", H.ff }); downs.push_back({ q + "down", width });
+                }
+                if (!(W.e_up = L.matrix(ups, width)) || !(W.e_down = L.matrix(downs, H.ff))) return false;
+                if (H.shared_ff > 0 && (!(W.ff_up = L.matrix({ { p + "mlp.shared.gate", H.shared_ff }, { p + "mlp.shared.up", H.shared_ff } }, width)) || !(W.ff_down = L.matrix({ { p + "mlp.shared.down", width } }, H.shared_ff)))) return false;
+            }
+            W.loaded = true;
+            continue;
+        }
         const int64_t hd = (int64_t) H.heads * H.dim, hv = (int64_t) H.heads * H.vdim;
         if (!(W.norm1 = L.vector(p + "norm1", width))) return false;
         if (H.mixer == PI_MIXER_LIGHTNING) {
@@ -140,10 +254,23 @@ llama_model * load_hybrid_model(const std::string & folder, const llama_model_pa
     pi_hparams & hp = m->hparams;
     // the registry of folder-described architectures (GGUF files name theirs in general.architecture, model.cpp)
     if (arch->str == "Fasovik") hp.arch = PI_ARCH_FASOVIK;
-    else return fail("architecture '" + arch->str + "' is not one this engine builds (Fasovik)");
+    else if (arch->str == "Vikarax") hp.arch = PI_ARCH_VIKARAX;
+    else return fail("architecture '" + arch->str + "' is not one this engine builds (Fasovik, Vikarax)");
     m->name = arch->str;
     double d;
     if (!int_at(cfg, "vocab", hp.n_vocab) || !int_at(cfg, "width", hp.n_embd) || hp.n_vocab < 1 || hp.n_embd < 1) return fail("'vocab' and 'width' must be positive integers");
+    if (hp.arch == PI_ARCH_VIKARAX) {
+        std::string what;
+        if (!read_vikarax_config(cfg, hp, what)) return fail(what);
+        m->hweights.resize((size_t) hp.n_layer);
+        if (!params.vocab_only) {
+            if (!m->st_file.open(folder + "/model.safetensors", err)) { fprintf(stderr, "llama_load_model_from_file: %s\n", err.c_str()); return nullptr; }
+            for (const auto & kv : m->st_file.tensors) { m->n_elements += (uint64_t) kv.second.elements(); m->n_bytes += kv.second.nbytes; }
+            const st_tensor * e = m->st_file.tensor("embed"), * h = m->st_file.tensor("head");
+            if (!e || e->shape != std::vector<int64_t>{ hp.n_vocab, hp.n_embd } || !h || h->shape != e->shape) return fail("tensors 'embed' and 'head' are missing or not [vocab][width]");
+        }
+        return m.release();
+    }
     if (!num_at(cfg, "embedding.scale", d)) return fail("no 'embedding.scale'");
     hp.embed_scale = (float) d;
     if (!num_at(cfg, "norm.eps", d)) return fail("no 'norm.eps'");
@@ -186,7 +313,7 @@ llama_model * load_hybrid_model(const std::string & folder, const llama_model_pa
             if (!int_at(jl, "mlp.router.experts", H.n_expert) || !int_at(jl, "mlp.router.identity", H.n_identity) || !int_at(jl, "mlp.router.top", H.top)) return fail(where + "mlp.router needs 'experts', 'identity', 'top'");
             if (H.n_expert > 0 && (!int_at(jl, "mlp.expert.ff", H.ff) || H.ff < 1)) return fail(where + "mlp.expert needs 'ff'");
             if (H.top < 1 || H.top > H.n_expert + H.n_identity) return fail(where + "'top' must lie between 1 and the number of router outputs");
-            H.has_mlp = true;
+            H.has_mlp = true; H.mlp = PI_MLP_MOE_RELU_SQR;
         }
         hp.hybrid.push_back(std::move(H));
     }

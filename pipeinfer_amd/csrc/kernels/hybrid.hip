@@ -5,6 +5,8 @@
 //   k_linear_attention   per head S <- lambda * S + k v^T, o = S^T q over a run of tokens of one sequence; S lives in HBM per (slot, head) between calls
 //   k_latent_attention   attention over a shared low-rank latent c: the key up-projection is folded into the query (q~ = W_uk^T q), the value up-projection applied to the
 //                        probability-weighted sum of latents — the cache is read once for all heads of a tile and K / V are never materialised; soft-max with a sink term
+//   k_layer_norm_mix     y = ((ca * a + cb * b) - mean) / sqrt(variance + eps) * w + bias;  out = [residual +] y   (the norm behind a sublayer with two branches)
+//   k_depth_mix          out = sum_j coef[j] * X_j over the stream's earlier states (a learned average over depth)
 //   k_moe_route          router logits, soft-max over all router outputs, bias-corrected top-k choice, weights = uncorrected scores
 //   k_moe_up / _down     the chosen experts of every token (gathered mat-vecs), identity experts pass their input through
 #include "ops_common.h"
@@ -101,6 +103,76 @@ extern "C" int pi_op_rms_scale(const float * x, int64_t x_stride, const float * 
     PI_CHECK_LAUNCH(); return 0;
 }
 
+// ---- layer norm (weight and bias) over one or the weighted sum of two inputs, optional residual ---------------------------------------------------------------
+// two passes over the row for the statistics (mean, then the mean of squared deviations), a third for the output: the row stays in L2 / registers' reach
+__global__ void __launch_bounds__(256) k_layer_norm_mix(const float * __restrict__ a, int64_t as, float ca, const float * __restrict__ b, int64_t bs, float cb, const float * __restrict__ w,
+                                                        const float * __restrict__ bias, float eps, int n, const float * __restrict__ res, int64_t rs, float * __restrict__ out, int64_t os,
+                                                        const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    __shared__ float red[4];
+    const int t = blockIdx.x;
+    const float * ar = a + (int64_t) t * as, * br = b ? b + (int64_t) t * bs : nullptr;
+    auto val = [&](int i) { const float v = ca * ar[i]; return br ? fmaf(cb, br[i], v) : v; };
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) sum += val(i);
+    const float mean = hy_block_sum(sum, red) / (float) n;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) { const float d = val(i) - mean; ss = fmaf(d, d, ss); }
+    const float inv = 1.0f / sqrtf(hy_block_sum(ss, red) / (float) n + eps);
+    for (int i = threadIdx.x; i < n; i += 256) {
+        float y = (val(i) - mean) * inv * w[i] + (bias ? bias[i] : 0.0f);
+        if (res) y = res[(int64_t) t * rs + i] + y;
+        out[(int64_t) t * os + i] = y;
+    }
+}
+extern "C" int pi_op_layer_norm_mix(const float * a, int64_t a_stride, float ca, const float * b, int64_t b_stride, float cb, const float * w_dev, const float * bias_dev, float eps, int n, int n_tok,
+                                    const float * residual, int64_t residual_stride, float * out, int64_t out_stride, void * stream) {
+    if (n_tok <= 0 || n <= 0) return 0;
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 4.0 * n * n_tok * (2.0 + (b ? 1 : 0) + (residual ? 1 : 0)), k_layer_norm_mix, dim3((unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, a, a_stride, ca, b, b_stride, cb,
+                 w_dev, bias_dev, eps, n, residual, residual_stride, out, out_stride, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// out[t][i] = sum_j coef[j] * hist[j][t][i], j ascending; hist: n_hist arrays [n_tok rows][n], `hist_stride` floats apart
+__global__ void __launch_bounds__(256) k_depth_mix(const float * __restrict__ hist, int64_t hist_stride, int n_hist, const float * __restrict__ coef, int n, float * __restrict__ out, int64_t os,
+                                                   const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float a = 0.0f;
+    for (int j = 0; j < n_hist; j++) a = fmaf(coef[j], hist[(int64_t) j * hist_stride + (int64_t) t * n + i], a);
+    out[(int64_t) t * os + i] = a;
+}
+extern "C" int pi_op_depth_mix(const float * hist, int64_t hist_stride, int n_hist, const float * coef_dev, int n, int n_tok, float * out, int64_t out_stride, void * stream) {
+    if (n_tok <= 0 || n <= 0 || n_hist <= 0) return 0;
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 4.0 * n * n_tok * (n_hist + 1.0), k_depth_mix, dim3((unsigned) ((n + 255) / 256), (unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, hist, hist_stride, n_hist, coef_dev, n,
+                 out, out_stride, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// x <- cap * tanh(x / cap) in place
+__global__ void k_softcap(float * __restrict__ x, int64_t n, float cap, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    for (int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t) gridDim.x * 256) x[i] = cap * tanhf(x[i] / cap);
+}
+extern "C" int pi_op_softcap(float * x, int64_t n, float cap, void * stream) {
+    if (n <= 0) return 0;
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * n, k_softcap, dim3((unsigned) std::max<int64_t>(1, std::min<int64_t>(4096, (n + 255) / 256))), dim3(256), 0, (hipStream_t) stream, x, n, cap, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// out[t][f] = in[t][f] * in[t][ff + f]  (a gated feed-forward whose gate and up rows are one matrix; the gate's activation ran in the projection's epilogue)
+__global__ void k_glu_mul(const float * __restrict__ in, int64_t is, int ff, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.y, f = blockIdx.x * 256 + threadIdx.x;
+    if (f < ff) out[(int64_t) t * os + f] = in[(int64_t) t * is + f] * in[(int64_t) t * is + ff + f];
+}
+extern "C" int pi_op_glu_mul(const float * in, int64_t in_stride, int ff, int n_tok, float * out, int64_t out_stride, void * stream) {
+    if (n_tok <= 0 || ff <= 0) return 0;
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 12.0 * ff * n_tok, k_glu_mul, dim3((unsigned) ((ff + 255) / 256), (unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, in, in_stride, ff, out, out_stride, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
 // ---- linear attention with a per-head decay -------------------------------------------------------------------------------------------------------
 // rec[t] = state slot of token t (| 1 << 30 on the first token of a sequence whose state starts from zero), tokens of one slot are consecutive.  Workgroup (head, column block,
 // piece): thread (column j, part sp of R) keeps S[i][j] for its DPT rows i in registers and walks the piece's tokens in order.
@@ -141,12 +213,14 @@ static __device__ __forceinline__ bool la_find_piece(const int * recs, int n_tok
     return false;
 }
 template <int DPT>
-__global__ void __launch_bounds__(256) k_linear_attention(const float * __restrict__ q, const float * __restrict__ k, const float * __restrict__ v, int64_t stride, int heads, int dim, int vdim, int R,
-                                                          const float * __restrict__ decay, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, int mode, float * __restrict__ scratch,
+__global__ void __launch_bounds__(256) k_linear_attention(const float * __restrict__ q, const float * __restrict__ k, const float * __restrict__ v, int64_t stride, int heads, int hpg, int dim, int vdim, int R,
+                                                          const float * __restrict__ decay, const float * __restrict__ tdecay, const float * __restrict__ tscale, int64_t tds, const float * __restrict__ skip,
+                                                          float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, int mode, float * __restrict__ scratch,
                                                           float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     extern __shared__ float lds[];                // q tile [LA_TB][dim] | k tile [LA_TB][dim] | v tile [LA_TB][cols] | the slot words of the pass [n_tok]
     __shared__ int seg[4], bnd[LA_MAXRUNS], nbnd; // seg: first token, length, slot word, last piece of its run
+    __shared__ float lam_t[LA_TB], sc_t[LA_TB];   // per token of the tile: decay and the factor on k v^T
     const int h = blockIdx.x, tid = threadIdx.x;
     int * recs = (int *) (lds + 2 * LA_TB * dim + LA_TB * (blockDim.x / R));
     for (int t = tid; t < n_tok; t += blockDim.x) recs[t] = rec[t];
@@ -164,7 +238,8 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
     const int cols = blockDim.x / R;
     const int j = blockIdx.y * cols + tid / R, sp = tid % R;
     const bool col_ok = j < vdim;
-    const float lam = decay[h];
+    const float lam = decay ? decay[h] : 1.0f, skp = skip ? skip[h] : 0.0f;
+    const int hq = h / hpg;                                            // the q / k head this head reads (hpg heads share one)
     float * S_hbm = state + ((int64_t) slot * heads + h) * dim * vdim;
     float * S_scr = scratch ? scratch + ((int64_t) blockIdx.z * heads + h) * dim * vdim : nullptr;
     const float * S_from = mode == 2 ? S_scr : mode == 1 || (word & LA_FRESH) ? nullptr : S_hbm;
@@ -181,9 +256,13 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
         __syncthreads();
         for (int idx = tid; idx < nt * dim; idx += blockDim.x) {
             const int tt = idx / dim, i = idx % dim;
-            const int64_t off = (int64_t) (first + t0 + tt) * stride + (int64_t) h * dim + i;
+            const int64_t off = (int64_t) (first + t0 + tt) * stride + (int64_t) hq * dim + i;
             if (mode != 1) qt[idx] = q[off];
             kt[idx] = k[off];
+        }
+        if (tid < nt) {
+            lam_t[tid] = tdecay ? tdecay[(int64_t) (first + t0 + tid) * tds + h] : lam;
+            sc_t[tid] = tscale ? tscale[(int64_t) (first + t0 + tid) * tds + h] : 1.0f;
         }
         for (int idx = tid; idx < nt * cols; idx += blockDim.x) {
             const int tt = idx / cols, jj = blockIdx.y * cols + idx % cols;
@@ -192,7 +271,7 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
         __syncthreads();
         if (mode == 1) {                                              // the state only
             for (int tt = 0; tt < nt; tt++) {
-                const float vj = vt[tt * cols + tid / R];
+                const float vj = vt[tt * cols + tid / R] * sc_t[tt], lam = lam_t[tt];
                 const float * kr = kt + tt * dim + sp * DPT;
 #pragma unroll
                 for (int ii = 0; ii < DPT; ii++) if (sp * DPT + ii < dim) S[ii] = fmaf(kr[ii], vj, lam * S[ii]);
@@ -200,7 +279,7 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
             continue;
         }
         for (int tt = 0; tt < nt; tt++) {
-            const float vj = vt[tt * cols + tid / R];
+            const float vraw = vt[tt * cols + tid / R], vj = vraw * sc_t[tt], lam = lam_t[tt];
             const float * kr = kt + tt * dim + sp * DPT, * qr = qt + tt * dim + sp * DPT;
             float o = 0.0f;
             if (dim4) {
@@ -222,7 +301,7 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
             if (R == 2) o += pi_partner<1>(o);
             else if (R == 4) { o += pi_partner<2>(o); o += pi_partner<1>(o); }
             else for (int d = R >> 1; d > 0; d >>= 1) o += __shfl_xor(o, d, PI_WAVE);
-            if (col_ok && sp == 0) out[(int64_t) (first + t0 + tt) * os + (int64_t) h * vdim + j] = o;
+            if (col_ok && sp == 0) out[(int64_t) (first + t0 + tt) * os + (int64_t) h * vdim + j] = fmaf(skp, vraw, o);
         }
     }
     float * S_to = mode == 1 ? S_scr : last ? S_hbm : nullptr;
@@ -232,32 +311,32 @@ __global__ void __launch_bounds__(256) k_linear_attention(const float * __restri
 }
 
 // grid (head, blocks over dim * vdim, run): scratch[piece] holds L_p coming in and S_in(p) going out
-__global__ void __launch_bounds__(256) k_linear_state_scan(int heads, int dim, int vdim, const float * __restrict__ decay, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
-                                                           float * __restrict__ scratch, const int32_t * __restrict__ abort_w) {
+__global__ void __launch_bounds__(256) k_linear_state_scan(int heads, int dim, int vdim, const float * __restrict__ decay, const float * __restrict__ tdecay, int64_t tds, const float * __restrict__ state,
+                                                           const int32_t * __restrict__ rec, int n_tok, float * __restrict__ scratch, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
-    __shared__ int seg[3], bnd[LA_MAXRUNS], nbnd; // seg: slot word, first piece ordinal, pieces of the run (0: no such run)
+    __shared__ int seg[4], bnd[LA_MAXRUNS], nbnd; // seg: slot word, first piece ordinal, pieces of the run (0: no such run), the run's first token
     extern __shared__ int recs[];                 // the slot words of the pass
     for (int t = threadIdx.x; t < n_tok; t += 256) recs[t] = rec[t];
     __syncthreads();
     const int n_runs = la_runs(recs, n_tok, bnd, &nbnd);
     if (threadIdx.x == 0) {
-        int ord = 0, nsub = 0, word = -1, sub0 = 0;
+        int ord = 0, nsub = 0, word = -1, sub0 = 0, tfirst = 0;
         for (int r = 0; r < n_runs; r++) {
             const int t = bnd[r], e = r + 1 < n_runs ? bnd[r + 1] : n_tok;
             const int ns = (e - t + LA_TB - 1) / LA_TB;
-            if (r == (int) blockIdx.z) { nsub = ns; word = recs[t]; sub0 = ord; break; }
+            if (r == (int) blockIdx.z) { nsub = ns; word = recs[t]; sub0 = ord; tfirst = t; break; }
             ord += ns;
         }
-        seg[0] = word; seg[1] = sub0; seg[2] = nsub;
+        seg[0] = word; seg[1] = sub0; seg[2] = nsub; seg[3] = tfirst;
     }
     __syncthreads();
-    const int word = seg[0], sub0 = seg[1], nsub = seg[2];
+    const int word = seg[0], sub0 = seg[1], nsub = seg[2], tfirst = seg[3];
     if (nsub == 0 || word < 0) return;
     const int h = blockIdx.x, slot = word & ~LA_FRESH;
     const int64_t per = (int64_t) dim * vdim, idx = (int64_t) blockIdx.y * 256 + threadIdx.x;
     if (idx >= per) return;
     float lp = 1.0f;                                                   // lambda^LA_TB: every piece but a run's last has LA_TB tokens
-    for (int i = 0; i < LA_TB; i++) lp *= decay[h];
+    if (!tdecay) for (int i = 0; i < LA_TB; i++) lp *= decay[h];
     float run = (word & LA_FRESH) ? 0.0f : state[((int64_t) slot * heads + h) * per + idx];
     for (int p0 = 0; p0 < nsub; p0 += 8) {                             // eight pieces at a time: their loads are in flight together, then the chain runs on registers
         float lpart[8];
@@ -265,7 +344,15 @@ __global__ void __launch_bounds__(256) k_linear_state_scan(int heads, int dim, i
         for (int i = 0; i < 8; i++) lpart[i] = p0 + i < nsub - 1 ? scratch[((int64_t) (sub0 + p0 + i) * heads + h) * per + idx] : 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; i++)
-            if (p0 + i < nsub) { scratch[((int64_t) (sub0 + p0 + i) * heads + h) * per + idx] = run; run = fmaf(lp, run, lpart[i]); }
+            if (p0 + i < nsub) {
+                scratch[((int64_t) (sub0 + p0 + i) * heads + h) * per + idx] = run;
+                if (tdecay && p0 + i < nsub - 1) {                     // per-token decays: the product over the piece's tokens
+                    lp = 1.0f;
+                    const float * td = tdecay + (int64_t) (tfirst + (p0 + i) * LA_TB) * tds + h;
+                    for (int j = 0; j < LA_TB; j++) lp *= td[(int64_t) j * tds];
+                }
+                run = fmaf(lp, run, lpart[i]);
+            }
     }
 }
 
@@ -275,7 +362,15 @@ extern "C" size_t pi_op_linear_attention_scratch_floats(int heads, int dim, int 
 }
 extern "C" int pi_op_linear_attention(const float * q, const float * k, const float * v, int64_t stride, int heads, int dim, int vdim, const float * decay_dev, float * state_dev,
                                       const int32_t * rec_dev, int n_tok, int max_segments, float * scratch_dev, size_t scratch_floats, float * out, int64_t out_stride, void * stream) {
+    return pi_op_linear_attention_ex(q, k, v, stride, heads, heads, dim, vdim, decay_dev, nullptr, nullptr, 0, nullptr, state_dev, rec_dev, n_tok, max_segments, scratch_dev, scratch_floats, out, out_stride, stream);
+}
+extern "C" int pi_op_linear_attention_ex(const float * q, const float * k, const float * v, int64_t stride, int heads, int qk_heads, int dim, int vdim, const float * decay_dev, const float * tdecay_dev,
+                                         const float * tscale_dev, int64_t t_stride, const float * skip_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int max_segments, float * scratch_dev,
+                                         size_t scratch_floats, float * out, int64_t out_stride, void * stream) {
     if (n_tok <= 0) return 0;
+    if (qk_heads < 1 || heads % qk_heads) { pi_set_error("pi_op_linear_attention: %d heads do not divide over %d query / key heads", heads, qk_heads); return -1; }
+    if (!decay_dev && !tdecay_dev) { pi_set_error("pi_op_linear_attention: neither per-head nor per-token decays were given"); return -1; }
+    const int hpg = heads / qk_heads;
     if (dim <= 0 || vdim <= 0 || heads <= 0 || dim > 1024) { pi_set_error("pi_op_linear_attention: head sizes %d x %d outside the kernel's range (key width <= 1024)", dim, vdim); return -1; }
     if (max_segments > LA_MAXRUNS) { pi_set_error("pi_op_linear_attention: at most %d sequences in a pass", LA_MAXRUNS); return -1; }
     const int dpt = dim <= 8 ? 8 : dim <= 16 ? 16 : 32;                // state values a thread keeps in registers (more would spill in the token loop)
@@ -290,13 +385,13 @@ extern "C" int pi_op_linear_attention(const float * q, const float * k, const fl
     const double bytes = 4.0 * n_tok * heads * (2.0 * dim + 2.0 * vdim) + 8.0 * heads * dim * vdim;
     hipStream_t s = (hipStream_t) stream;
     const int nta = std::min(n_tok, PI_KT_MAXNT - 1);
-#define LA_GO(D, MODE) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, bytes, k_linear_attention<D>, grid, dim3(threads), lds, s, q, k, v, stride, heads, dim, vdim, R, decay_dev, state_dev, rec_dev, n_tok, MODE, scratch_dev, out, out_stride, pi_abort_word())
+#define LA_GO(D, MODE) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, bytes, k_linear_attention<D>, grid, dim3(threads), lds, s, q, k, v, stride, heads, hpg, dim, vdim, R, decay_dev, tdecay_dev, tscale_dev, t_stride, skip_dev, state_dev, rec_dev, n_tok, MODE, scratch_dev, out, out_stride, pi_abort_word())
 #define LA_ANY(MODE) do { if (dpt == 8) LA_GO(8, MODE); else if (dpt == 16) LA_GO(16, MODE); else LA_GO(32, MODE); } while (0)
     if (!pieces) { LA_ANY(0); PI_CHECK_LAUNCH(); return 0; }
     LA_ANY(1);
     PI_CHECK_LAUNCH();
     PI_KT_LAUNCH(PI_KT_ATT, 0, nta, 12.0 * gz * heads * dim * vdim, k_linear_state_scan, dim3((unsigned) heads, (unsigned) (((int64_t) dim * vdim + 255) / 256), (unsigned) std::max(1, std::min(n_tok, max_segments))), dim3(256), (size_t) 4 * n_tok, s,
-                 heads, dim, vdim, decay_dev, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word());
+                 heads, dim, vdim, decay_dev, tdecay_dev, t_stride, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word());
     PI_CHECK_LAUNCH();
     LA_ANY(2);
 #undef LA_ANY
@@ -639,11 +734,13 @@ extern "C" int pi_op_latent_attention(const float * q, int64_t q_stride, const f
 
 // ---- routed feed-forward ------------------------------------------------------------------------------------------------------------------------------
 // one workgroup per token: logits of all router outputs (a wave per output), soft-max, choice = score + correction, `top` rounds of arg-max (lowest index wins a tie)
+// n_groups > 0: the scores are sigmoid(logit), the outputs form n_groups equal groups of neighbours, a group's score is the sum of its two largest scores and only outputs of the
+// `keep` best groups can be chosen (by their own score; lowest index wins a tie, among groups as among outputs)
 __global__ void __launch_bounds__(256) k_moe_route(const uint16_t * __restrict__ router, int64_t width, int n_out, const float * __restrict__ corr, const float * __restrict__ x, int64_t xs,
-                                                   int top, int exact, int vec, int32_t * __restrict__ sel, float * __restrict__ selw, const int32_t * __restrict__ abort_w) {
+                                                   int top, int exact, int vec, int n_groups, int keep, int32_t * __restrict__ sel, float * __restrict__ selw, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
-    extern __shared__ float z[];                  // [n_out] logits -> scores | [n_out] choice
-    float * ch = z + n_out;
+    extern __shared__ float z[];                  // [n_out] logits -> scores | [n_out] choice | [n_groups] group scores
+    float * ch = z + n_out, * gsc = ch + n_out;
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float * xr = x + (int64_t) t * xs;
     for (int e = wave; e < n_out; e += 4) {
@@ -652,6 +749,26 @@ __global__ void __launch_bounds__(256) k_moe_route(const uint16_t * __restrict__
     }
     __syncthreads();
     if (wave != 0) return;
+    if (n_groups > 0) {
+        const int per = n_out / n_groups;
+        for (int e = lane; e < n_out; e += 64) { z[e] = 1.0f / (1.0f + expf(-z[e])); ch[e] = -INFINITY; }
+        for (int g = lane; g < n_groups; g += 64) {
+            float b0 = -INFINITY, b1 = -INFINITY;
+            for (int e = g * per; e < (g + 1) * per; e++) { const float v = z[e]; if (v > b0) { b1 = b0; b0 = v; } else if (v > b1) b1 = v; }
+            gsc[g] = b1 == -INFINITY ? b0 : b0 + b1;
+        }
+        for (int kk = 0; kk < keep; kk++) {
+            float bv = -INFINITY; int bi = 0x7fffffff;
+            for (int g = lane; g < n_groups; g += 64) { const float c = gsc[g]; if (c > bv || (c == bv && g < bi)) { bv = c; bi = g; } }
+            for (int d = 32; d > 0; d >>= 1) {
+                const float ov = __shfl_xor(bv, d, PI_WAVE); const int oi = __shfl_xor(bi, d, PI_WAVE);
+                if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+            }
+            if (bi == 0x7fffffff) break;
+            for (int e = bi * per + lane; e < (bi + 1) * per; e += 64) ch[e] = z[e];
+            if (lane == 0) gsc[bi] = -INFINITY;
+        }
+    } else {
     float m = -INFINITY;
     for (int e = lane; e < n_out; e += 64) m = fmaxf(m, z[e]);
     m = pi_wave_max(m);
@@ -659,6 +776,7 @@ __global__ void __launch_bounds__(256) k_moe_route(const uint16_t * __restrict__
     for (int e = lane; e < n_out; e += 64) { const float p = expf(z[e] - m); z[e] = p; l += p; }
     l = pi_lanes_sum<64>(l);
     for (int e = lane; e < n_out; e += 64) { z[e] = z[e] / l; ch[e] = z[e] + corr[e]; }
+    }
     for (int kk = 0; kk < top; kk++) {
         float bv = -INFINITY; int bi = 0x7fffffff;
         for (int e = lane; e < n_out; e += 64) { const float c = ch[e]; if (c > bv || (c == bv && e < bi)) { bv = c; bi = e; } }
@@ -671,15 +789,22 @@ __global__ void __launch_bounds__(256) k_moe_route(const uint16_t * __restrict__
     }
 }
 
-// up[t][kk][f] = relu(W_up[e] x_t)^2 for the kk-th chosen expert e of token t (nothing for identity experts); a wave per row f
+// up[t][kk][f] = relu(W_up[e] x_t)^2 for the kk-th chosen expert e of token t (nothing for identity experts); a wave per row f.
+// glu: an expert's first matrix holds 2 * ff rows [gate | up] and up[t][kk][f] = silu(gate_f . x) * (up_f . x)
 __global__ void __launch_bounds__(256) k_moe_up(const uint16_t * __restrict__ wup, int64_t width, int ff, int n_exp, const float * __restrict__ x, int64_t xs, const int32_t * __restrict__ sel,
-                                                int top, int exact, int vec, float * __restrict__ up, const int32_t * __restrict__ abort_w) {
+                                                int top, int exact, int vec, int glu, float * __restrict__ up, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 0)) return;
     const int lane = threadIdx.x & 63, f = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int slot = blockIdx.y, e = sel[slot];
     if (f >= ff || e >= n_exp) return;
     const int t = slot / top;
     const float * xr = x + (int64_t) t * xs;
+    if (glu) {
+        const float g = pi_lanes_sum<64>(hy_dot_lane(wup + ((int64_t) e * 2 * ff + f) * width, xr, width, lane, exact != 0, vec != 0));
+        const float u = pi_lanes_sum<64>(hy_dot_lane(wup + ((int64_t) e * 2 * ff + ff + f) * width, xr, width, lane, exact != 0, vec != 0));
+        if (lane == 0) up[(int64_t) slot * ff + f] = g / (1.0f + expf(-g)) * u;
+        return;
+    }
     const float a = pi_lanes_sum<64>(hy_dot_lane(wup + ((int64_t) e * ff + f) * width, xr, width, lane, exact != 0, vec != 0));
     if (lane == 0) { const float r = fmaxf(a, 0.0f); up[(int64_t) slot * ff + f] = r * r; }
 }
@@ -703,29 +828,43 @@ __global__ void __launch_bounds__(256) k_moe_down(const uint16_t * __restrict__ 
     if (lane == 0) out[(int64_t) t * os + n] = acc;
 }
 
-extern "C" int pi_op_moe_route(const pi_weight * router, const float * correction_dev, const float * x, int64_t x_stride, int n_tok, int top, int exact, int32_t * sel_dev, float * selw_dev, void * stream) {
+static int moe_route_launch(const pi_weight * router, const float * correction_dev, const float * x, int64_t x_stride, int n_tok, int top, int exact, int n_groups, int keep, int32_t * sel_dev, float * selw_dev, void * stream) {
     if (n_tok <= 0) return 0;
     if (!router || router->type != PI_BF16 || top < 1 || top > router->ne1 || router->ne1 > 8192) { pi_set_error("pi_op_moe_route: a bfloat16 router of at most 8192 outputs and 1 <= top <= outputs are required"); return -1; }
-    PI_KT_LAUNCH(PI_KT_OTHER, PI_BF16, 1, 2.0 * router->ne0 * router->ne1 + 4.0 * n_tok * router->ne0, k_moe_route, dim3((unsigned) n_tok), dim3(256), (size_t) 8 * router->ne1, (hipStream_t) stream,
+    PI_KT_LAUNCH(PI_KT_OTHER, PI_BF16, 1, 2.0 * router->ne0 * router->ne1 + 4.0 * n_tok * router->ne0, k_moe_route, dim3((unsigned) n_tok), dim3(256), (size_t) 8 * router->ne1 + (size_t) 4 * std::max(n_groups, 1), (hipStream_t) stream,
                  (const uint16_t *) router->p0, router->ne0, (int) router->ne1, correction_dev, x, x_stride, top, exact,
-                 (int) (router->ne0 % 8 == 0 && ((uintptr_t) router->p0 % 16) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0), sel_dev, selw_dev, pi_abort_word());
+                 (int) (router->ne0 % 8 == 0 && ((uintptr_t) router->p0 % 16) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0), n_groups, keep, sel_dev, selw_dev, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
+}
+extern "C" int pi_op_moe_route(const pi_weight * router, const float * correction_dev, const float * x, int64_t x_stride, int n_tok, int top, int exact, int32_t * sel_dev, float * selw_dev, void * stream) {
+    return moe_route_launch(router, correction_dev, x, x_stride, n_tok, top, exact, 0, 0, sel_dev, selw_dev, stream);
+}
+extern "C" int pi_op_moe_route_groups(const pi_weight * router, const float * x, int64_t x_stride, int n_tok, int top, int n_groups, int keep, int exact, int32_t * sel_dev, float * selw_dev, void * stream) {
+    if (!router || n_groups < 1 || router->ne1 % n_groups || keep < 1 || keep > n_groups || (int64_t) keep * (router->ne1 / n_groups) < top) {
+        pi_set_error("pi_op_moe_route_groups: the router's outputs must divide into the groups, and the kept groups must hold at least `top` outputs"); return -1;
+    }
+    return moe_route_launch(router, nullptr, x, x_stride, n_tok, top, exact, n_groups, keep, sel_dev, selw_dev, stream);
 }
 // wup: [n_exp * ff][width], wdown: [n_exp * width][ff] (the experts' matrices one after the other); up_dev: scratch [n_tok][top][ff]
 extern "C" int pi_op_moe_experts(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, const float * x, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
                                  int exact, float * up_dev, float * out, int64_t out_stride, void * stream) {
+    return pi_op_moe_experts_act(wup, wdown, n_exp, ff, 0, x, x_stride, sel_dev, selw_dev, n_tok, top, exact, up_dev, out, out_stride, stream);
+}
+extern "C" int pi_op_moe_experts_act(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, int glu, const float * x, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
+                                     int exact, float * up_dev, float * out, int64_t out_stride, void * stream) {
     if (n_tok <= 0) return 0;
+    const int upr = glu ? 2 : 1;                                       // rows of an expert's first matrix, in units of ff
     hipStream_t s = (hipStream_t) stream;
     int64_t width = 0;
     if (n_exp > 0) {
-        if (!wup || !wdown || wup->type != PI_BF16 || wdown->type != PI_BF16 || wup->ne1 != (int64_t) n_exp * ff || wdown->ne0 != ff || wdown->ne1 != (int64_t) n_exp * wup->ne0) {
-            pi_set_error("pi_op_moe_experts: expert matrices must be bfloat16 [experts * ff][width] and [experts * width][ff]"); return -1;
+        if (!wup || !wdown || wup->type != PI_BF16 || wdown->type != PI_BF16 || wup->ne1 != (int64_t) n_exp * ff * upr || wdown->ne0 != ff || wdown->ne1 != (int64_t) n_exp * wup->ne0) {
+            pi_set_error("pi_op_moe_experts: expert matrices must be bfloat16 [experts * ff (twice with a gate)][width] and [experts * width][ff]"); return -1;
         }
         width = wup->ne0;
-        const double b_up = std::min<double>(n_tok * top, n_exp) * 2.0 * ff * width + 4.0 * n_tok * (width + (double) top * ff);
+        const double b_up = std::min<double>(n_tok * top, n_exp) * 2.0 * upr * ff * width + 4.0 * n_tok * (width + (double) top * ff);
         PI_KT_LAUNCH(PI_KT_MATVEC, PI_BF16, std::min(n_tok, PI_KT_MAXNT - 1), b_up, k_moe_up, dim3((unsigned) ((ff + 3) / 4), (unsigned) (n_tok * top)), dim3(256), 0, s,
                      (const uint16_t *) wup->p0, width, ff, n_exp, x, x_stride, sel_dev, top, exact,
-                     (int) (width % 8 == 0 && ((uintptr_t) wup->p0 % 16) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0), up_dev, pi_abort_word());
+                     (int) (width % 8 == 0 && ((uintptr_t) wup->p0 % 16) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0), glu, up_dev, pi_abort_word());
         PI_CHECK_LAUNCH();
     } else width = out_stride;
     const double b_dn = std::min<double>(n_tok * top, std::max(n_exp, 1)) * 2.0 * ff * width + 4.0 * n_tok * (width + (double) top * ff);
@@ -768,14 +907,21 @@ __global__ void __launch_bounds__(256) k_moe_group(const int32_t * __restrict__ 
 }
 
 // acc[j] += W[rows j*16 + (l % 16)][k] * B[slot (l % 16)][k] over K (K % 8 == 0); brow: this lane's B row (nullptr: zeros), wrow[j]: this lane's A rows (nullptr: zeros)
-static __device__ __forceinline__ void hy_mfma_rows(const uint16_t * const wrow[4], const float * brow, int64_t K, int kb, hy_f32x4 acc[4]) {
+// glu_off > 0: the B value at k is silu(brow[k]) * brow[glu_off + k] (a gated hidden layer whose two halves were stored raw)
+static __device__ __forceinline__ void hy_mfma_rows(const uint16_t * const wrow[4], const float * brow, int64_t K, int kb, hy_f32x4 acc[4], int64_t glu_off = 0) {
     for (int64_t k0 = 0; k0 < K; k0 += 32) {
         const int64_t k = k0 + kb * 8;
         const bool k_ok = k < K;
         hy_u16x8 b = hy_u16x8{0, 0, 0, 0, 0, 0, 0, 0};
         if (k_ok && brow) {
             const float4 v0 = *(const float4 *) (brow + k), v1 = *(const float4 *) (brow + k + 4);
-            const float f[8] = { v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w };
+            float f[8] = { v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w };
+            if (glu_off > 0) {
+                const float4 u0 = *(const float4 *) (brow + glu_off + k), u1 = *(const float4 *) (brow + glu_off + k + 4);
+                const float uf[8] = { u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w };
+#pragma unroll
+                for (int i = 0; i < 8; i++) f[i] = f[i] / (1.0f + expf(-f[i])) * uf[i];
+            }
 #pragma unroll
             for (int i = 0; i < 8; i++) { const uint32_t u = __float_as_uint(f[i]); b[i] = (uint16_t) ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16); }
         }
@@ -788,10 +934,11 @@ static __device__ __forceinline__ void hy_mfma_rows(const uint16_t * const wrow[
     }
 }
 
-// UP: B rows are the tokens' inputs x[slot / top], A rows W_up[e], out up[slot][f] = relu(.)^2;  !UP: B rows up[slot] (K = ff), A rows W_down[e], out dn[slot][n]
+// UP: B rows are the tokens' inputs x[slot / top], A rows W_up[e], out up[slot][f] = relu(.)^2;  !UP: B rows up[slot] (K = ff), A rows W_down[e], out dn[slot][n].
+// glu: UP leaves the 2 * ff rows [gate | up] of an expert raw, !UP forms silu(gate) * up while it reads them (bs = 2 * ff, K = ff)
 template <bool UP>
 __global__ void __launch_bounds__(256) k_moe_mfma(const uint16_t * __restrict__ W, int64_t K, int rows, const float * __restrict__ B, int64_t bs, int top, const int32_t * __restrict__ idx,
-                                                  int max_tiles, float * __restrict__ out, const int32_t * __restrict__ abort_w) {
+                                                  int max_tiles, int glu, float * __restrict__ out, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 1)) return;
     const int tile = blockIdx.y;
     if (tile >= idx[0]) return;
@@ -809,14 +956,14 @@ __global__ void __launch_bounds__(256) k_moe_mfma(const uint16_t * __restrict__ 
     hy_f32x4 acc[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[j] = hy_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    hy_mfma_rows(wrow, brow, K, kb, acc);
+    hy_mfma_rows(wrow, brow, K, kb, acc, !UP && glu ? K : 0);
     if (slot < 0) return;
 #pragma unroll
     for (int j = 0; j < 4; j++)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int row = n0 + j * 16 + kb * 4 + r;
-            if (row < rows) { float v = acc[j][r]; if (UP) { v = fmaxf(v, 0.0f); v *= v; } out[(int64_t) slot * rows + row] = v; }
+            if (row < rows) { float v = acc[j][r]; if (UP && !glu) { v = fmaxf(v, 0.0f); v *= v; } out[(int64_t) slot * rows + row] = v; }
         }
 }
 
@@ -837,7 +984,8 @@ __global__ void __launch_bounds__(256) k_moe_combine(const float * __restrict__ 
 // ints of index scratch the grouped path needs for a pass of n_tok tokens
 extern "C" size_t pi_op_moe_grouped_index_ints(int n_tok, int top, int n_exp) { const int ns = n_tok * top; return (size_t) 1 + 3 * (size_t) moe_max_tiles(ns, n_exp) + (size_t) ns; }
 // whether a pass of this shape takes the grouped matrix-core path (otherwise pi_op_moe_experts: gathered mat-vecs)
-extern "C" int pi_op_moe_grouped_ok(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, int n_tok, int top, int exact) {
+extern "C" int pi_op_moe_grouped_ok(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, int glu, int n_tok, int top, int exact) {
+    (void) glu;
     static const int min_slots = getenv("PI_MOE_GROUPED_MIN") ? atoi(getenv("PI_MOE_GROUPED_MIN")) : 32;
     return !exact && n_exp > 0 && n_exp <= MOE_GROUP_MAX_EXPERTS && wup && wdown && n_tok * top >= min_slots && wup->ne0 % 8 == 0 && ff % 8 == 0 &&
            ((uintptr_t) wup->p0 % 16) == 0 && ((uintptr_t) wdown->p0 % 16) == 0;
@@ -845,21 +993,27 @@ extern "C" int pi_op_moe_grouped_ok(const pi_weight * wup, const pi_weight * wdo
 // up_dev: [n_tok * top][ff], dn_dev: [n_tok * top][width], idx_dev: pi_op_moe_grouped_index_ints ints
 extern "C" int pi_op_moe_experts_grouped(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, const float * x, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
                                          float * up_dev, float * dn_dev, int32_t * idx_dev, float * out, int64_t out_stride, void * stream) {
-    if (!pi_op_moe_grouped_ok(wup, wdown, n_exp, ff, n_tok, top, 0)) { pi_set_error("pi_op_moe_experts_grouped: this shape takes pi_op_moe_experts"); return -1; }
-    if (wup->type != PI_BF16 || wdown->type != PI_BF16 || wup->ne1 != (int64_t) n_exp * ff || wdown->ne0 != ff || wdown->ne1 != (int64_t) n_exp * wup->ne0 || x_stride % 4 || ((uintptr_t) x % 16)) {
+    return pi_op_moe_experts_grouped_act(wup, wdown, n_exp, ff, 0, x, x_stride, sel_dev, selw_dev, n_tok, top, up_dev, dn_dev, idx_dev, out, out_stride, stream);
+}
+// glu: w_up holds [gate | up] per expert (2 * ff rows) and up_dev is [n_tok * top][2 * ff]
+extern "C" int pi_op_moe_experts_grouped_act(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, int glu, const float * x, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
+                                             float * up_dev, float * dn_dev, int32_t * idx_dev, float * out, int64_t out_stride, void * stream) {
+    if (!pi_op_moe_grouped_ok(wup, wdown, n_exp, ff, glu, n_tok, top, 0)) { pi_set_error("pi_op_moe_experts_grouped: this shape takes pi_op_moe_experts"); return -1; }
+    const int upr = glu ? 2 : 1;
+    if (wup->type != PI_BF16 || wdown->type != PI_BF16 || wup->ne1 != (int64_t) n_exp * ff * upr || wdown->ne0 != ff || wdown->ne1 != (int64_t) n_exp * wup->ne0 || x_stride % 4 || ((uintptr_t) x % 16)) {
         pi_set_error("pi_op_moe_experts_grouped: expert matrices must be bfloat16 [experts * ff][width] and [experts * width][ff], inputs 16-byte aligned rows"); return -1;
     }
     hipStream_t s = (hipStream_t) stream;
     const int64_t width = wup->ne0;
     const int ns = n_tok * top, mt = moe_max_tiles(ns, n_exp), nta = std::min(n_tok, PI_KT_MAXNT - 1);
-    const double wbytes = std::min<double>(ns, n_exp) * 2.0 * ff * width;
+    const double wbytes = std::min<double>(ns, n_exp) * 2.0 * ff * width * (glu ? 1.5 : 1.0);
     PI_KT_LAUNCH(PI_KT_OTHER, PI_BF16, 1, 8.0 * ns, k_moe_group, dim3(1), dim3(256), 0, s, sel_dev, ns, n_exp, mt, idx_dev, pi_abort_word());
     PI_CHECK_LAUNCH();
-    PI_KT_LAUNCH(PI_KT_MMQ, PI_BF16, nta, wbytes + 4.0 * ns * (width + ff), k_moe_mfma<true>, dim3((unsigned) ((ff + 63) / 64), (unsigned) mt), dim3(256), 0, s,
-                 (const uint16_t *) wup->p0, width, ff, x, x_stride, top, idx_dev, mt, up_dev, pi_abort_word());
+    PI_KT_LAUNCH(PI_KT_MMQ, PI_BF16, nta, wbytes + 4.0 * ns * (width + ff), k_moe_mfma<true>, dim3((unsigned) ((ff * upr + 63) / 64), (unsigned) mt), dim3(256), 0, s,
+                 (const uint16_t *) wup->p0, width, ff * upr, x, x_stride, top, idx_dev, mt, glu, up_dev, pi_abort_word());
     PI_CHECK_LAUNCH();
     PI_KT_LAUNCH(PI_KT_MMQ, PI_BF16, nta, wbytes + 4.0 * ns * (width + ff), k_moe_mfma<false>, dim3((unsigned) ((width + 63) / 64), (unsigned) mt), dim3(256), 0, s,
-                 (const uint16_t *) wdown->p0, (int64_t) ff, (int) width, up_dev, (int64_t) ff, top, idx_dev, mt, dn_dev, pi_abort_word());
+                 (const uint16_t *) wdown->p0, (int64_t) ff, (int) width, up_dev, (int64_t) ff * upr, top, idx_dev, mt, glu, dn_dev, pi_abort_word());
     PI_CHECK_LAUNCH();
     PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 4.0 * n_tok * width * (top + 2), k_moe_combine, dim3((unsigned) ((width + 255) / 256), (unsigned) n_tok), dim3(256), 0, s,
                  dn_dev, width, n_exp, top, x, x_stride, sel_dev, selw_dev, out, out_stride, pi_abort_word());

@@ -1,0 +1,297 @@
+// Operators of a mixer made of two branches that read the same input: attention with un-normalised sigmoid weights inside position chunks (grouped key / value heads,
+// normed and partly rotated queries and keys, unit-norm values, a per-head output gate), and a selective state-space recurrence with a short causal convolution in front
+// (state-space duality: per head S_t = a_t S_(t-1) + dt_t B_t x_t^T, y_t = S_t^T C_t + D x_t).  Everything here is fp32 in both precisions of the engine: norms, angles,
+// scores, weights, decays, step sizes, states.  The recurrence itself is pi_op_linear_attention_ex (hybrid.hip) with per-token decays and scales.
+//
+//   k_qkv_prepare        per token: RMS norm (shared per-head weight) + partial rotation of q and k, unit RMS of v; k and v go to the token's cache cell, the cell learns its position
+//   k_chunk_attention    out[t][h] = gate[t][h] * sum over visible cells c of sigmoid(q . K[c] * scale + bias[h]) V[c];  visible = the pass's mask bit AND position(c) >= start of t's chunk
+//   k_causal_conv        per channel: act(bias + sum_l w[l] * input(t - taps + 1 + l)), inputs before the pass come from the sequence's conv state (zeros for a fresh one)
+//   k_conv_state_update  the sequence's last taps - 1 inputs, for the next pass
+//   k_ssd_steps          dt = softplus(raw + bias), a = exp(-exp(A_log) * dt)
+//   k_gate_group_norm    u = y * silu(z); each of `groups` equal parts of u divided by its root mean square; * w
+#include "ops_common.h"
+#include "kernel_timing.h"
+
+#include <algorithm>
+#include <cmath>
+#include <vector>
+
+#define PM_FRESH (1 << 30)
+
+static __device__ __forceinline__ float pm_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
+static __device__ __forceinline__ float pm_block_sum(float v, float * red) {          // sum over the block's threads (every thread gets it); red: 4 floats, reusable after the call
+    v = pi_lanes_sum<64>(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float s = 0.0f;
+    for (int i = 0; i < (int) (blockDim.x >> 6); i++) s += red[i];
+    return s;
+}
+
+// ---- rotation table: cos / sin of p * base^(-2i / dims), angles formed in double on the host ------------------------------------------------------------
+struct pi_rotary_table { float2 * cs; int n_pos, half; };
+extern "C" void * pi_rotary_table_create(int n_pos, int dims, float base) {
+    if (n_pos < 1 || dims < 0 || (dims & 1)) { pi_set_error("pi_rotary_table_create: %d positions, %d rotated dimensions (an even number)", n_pos, dims); return nullptr; }
+    pi_rotary_table * t = new pi_rotary_table{ nullptr, n_pos, dims / 2 };
+    if (t->half == 0) return t;
+    std::vector<float2> h((size_t) n_pos * t->half);
+    for (int i = 0; i < t->half; i++) {
+        const double f = std::pow((double) base, -2.0 * i / dims);
+        for (int p = 0; p < n_pos; p++) { const double a = (double) p * f; h[(size_t) p * t->half + i] = make_float2((float) std::cos(a), (float) std::sin(a)); }
+    }
+    t->cs = (float2 *) pi_malloc(h.size() * sizeof(float2));
+    if (!t->cs || pi_memcpy_h2d(t->cs, h.data(), h.size() * sizeof(float2), nullptr) != 0 || pi_stream_sync(nullptr) != 0) { pi_free(t->cs); delete t; return nullptr; }
+    return t;
+}
+extern "C" int pi_rotary_table_positions(const void * table) { return table ? ((const pi_rotary_table *) table)->n_pos : 0; }
+extern "C" void pi_rotary_table_free(void * table) { pi_rotary_table * t = (pi_rotary_table *) table; if (t) { pi_free(t->cs); delete t; } }
+
+// ---- q / k / v of a pass ------------------------------------------------------------------------------------------------------------------------------
+// grid (token, head slot): slots [0, H) are query heads, [H, H + G) key heads, [H + G, H + 2G) value heads; one wave per slot
+__global__ void __launch_bounds__(64) k_qkv_prepare(const float * __restrict__ q, const float * __restrict__ k, const float * __restrict__ v, int64_t stride, const float * __restrict__ qw,
+                                                    const float * __restrict__ kw, float eps, int H, int G, int D, int V, const float2 * __restrict__ rot, int half, int n_pos,
+                                                    const int32_t * __restrict__ pos, float * __restrict__ q_out, int64_t qos, float * __restrict__ kc, float * __restrict__ vc,
+                                                    int32_t * __restrict__ cell_pos, const int32_t * __restrict__ dyn, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x, slot = blockIdx.y, lane = threadIdx.x;
+    const int cell = pi_cell_of(dyn, 0, t);
+    const int p = pos[t];
+    if (slot == 0 && lane == 0) cell_pos[cell] = p;
+    if (slot >= H + G) {                                              // a value head: divided by its root mean square, no weight
+        const int g = slot - H - G;
+        const float * src = v + (int64_t) t * stride + (int64_t) g * V;
+        float ss = 0.0f;
+        for (int i = lane; i < V; i += 64) ss = fmaf(src[i], src[i], ss);
+        const float inv = 1.0f / sqrtf(pi_lanes_sum<64>(ss) / (float) V + eps);
+        float * dst = vc + ((int64_t) cell * G + g) * V;
+        for (int i = lane; i < V; i += 64) dst[i] = src[i] * inv;
+        return;
+    }
+    const bool is_q = slot < H;
+    const int h = is_q ? slot : slot - H;
+    const float * src = (is_q ? q : k) + (int64_t) t * stride + (int64_t) h * D;
+    const float * w = is_q ? qw : kw;
+    float * dst = is_q ? q_out + (int64_t) t * qos + (int64_t) h * D : kc + ((int64_t) cell * G + h) * D;
+    float ss = 0.0f;
+    for (int i = lane; i < D; i += 64) ss = fmaf(src[i], src[i], ss);
+    const float inv = 1.0f / sqrtf(pi_lanes_sum<64>(ss) / (float) D + eps);
+    const float2 * cs = rot + (int64_t) min(p, n_pos - 1) * half;
+    for (int i = lane; i < D; i += 64) {
+        float y = src[i] * inv * w[i];
+        if (i < 2 * half) {                                           // dimension i pairs with i + half (i < half) or i - half
+            const int j = i < half ? i + half : i - half, f = i < half ? i : i - half;
+            const float o = src[j] * inv * w[j];
+            const float2 c = cs[f];
+            y = i < half ? y * c.x - o * c.y : y * c.x + o * c.y;
+        }
+        dst[i] = y;
+    }
+}
+
+extern "C" int pi_op_qkv_prepare(const float * q, const float * k, const float * v, int64_t stride, const float * q_norm_w, const float * k_norm_w, float eps, int heads, int kv_heads, int dim, int vdim,
+                                 const void * rotary_table, const int32_t * pos_dev, int n_tok, float * q_out, int64_t q_out_stride, float * k_cache, float * v_cache, int32_t * cell_pos_dev,
+                                 const int32_t * dyn_dev, void * stream) {
+    if (n_tok <= 0) return 0;
+    const pi_rotary_table * rt = (const pi_rotary_table *) rotary_table;
+    if (!rt || 2 * rt->half > dim) { pi_set_error("pi_op_qkv_prepare: a rotation table over at most %d dimensions is required", dim); return -1; }
+    if (heads < 1 || kv_heads < 1 || heads % kv_heads) { pi_set_error("pi_op_qkv_prepare: %d query heads do not divide over %d key / value heads", heads, kv_heads); return -1; }
+    if (!dyn_dev || !cell_pos_dev) { pi_set_error("pi_op_qkv_prepare: the pass's cell table and the cells' position array are required"); return -1; }
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * n_tok * ((double) heads * dim + (double) kv_heads * (dim + vdim)), k_qkv_prepare, dim3((unsigned) n_tok, (unsigned) (heads + 2 * kv_heads)), dim3(64), 0, (hipStream_t) stream,
+                 q, k, v, stride, q_norm_w, k_norm_w, eps, heads, kv_heads, dim, vdim, rt->cs, rt->half, rt->n_pos, pos_dev, q_out, q_out_stride, k_cache, v_cache, cell_pos_dev, dyn_dev, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// ---- attention with sigmoid weights inside chunks ---------------------------------------------------------------------------------------------------------
+// grid (token, key / value head): the workgroup serves the `hpg` query heads of its key head.  The cells are walked 256 at a time; the visible ones of a block are compacted
+// in cell order (so that the sum has one order whatever the launch), their key rows staged in LDS 64 at a time.  Scores: thread (cell, query head); output: thread (query
+// head, value column), value rows read from the cache along the columns.
+#define CA_TILE 64
+#define CA_MAXOUT 16                              // outputs (query head, value column) a thread accumulates: hpg * vdim <= 256 * CA_MAXOUT
+__global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * __restrict__ kc, const float * __restrict__ vc, const int32_t * __restrict__ cell_pos,
+                                                         const uint32_t * __restrict__ mask, const int32_t * __restrict__ pos, const float * __restrict__ hbias, const float * __restrict__ gate, int64_t gs, int gate_act,
+                                                         float scale, int chunk, int H, int G, int D, int V, int n_kv_arg, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
+                                                         const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w, 5)) return;
+    extern __shared__ float lds[];                // q [hpg][D] | key tile [CA_TILE][D + 1] | weights [CA_TILE][hpg]
+    __shared__ int list[256], wcnt[4];
+    const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hpg = H / G, h0 = g * hpg, DP = D + 1;
+    float * qsh = lds, * ksh = qsh + hpg * D, * wsh = ksh + CA_TILE * DP;
+    const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg);
+    const int words = (n_kv_arg + 31) / 32;
+    const uint32_t * mrow = mask + (int64_t) t * words;
+    const int p = pos[t];
+    const int first_pos = chunk > 0 ? p / chunk * chunk : 0;
+    for (int i = tid; i < hpg * D; i += 256) qsh[i] = q[(int64_t) t * qs + (int64_t) h0 * D + i];
+    float acc[CA_MAXOUT];
+#pragma unroll
+    for (int i = 0; i < CA_MAXOUT; i++) acc[i] = 0.0f;
+    const int n_out = hpg * V;
+    for (int c0 = 0; c0 < n_kv; c0 += 256) {
+        const int c = c0 + tid;
+        bool vis = false;
+        if (c < n_kv && ((mrow[c >> 5] >> (c & 31)) & 1u)) vis = cell_pos[c] >= first_pos;
+        const unsigned long long b = __ballot(vis);
+        __syncthreads();                          // (the previous block's list and tiles are no longer read)
+        if (lane == 0) wcnt[wave] = __popcll(b);
+        __syncthreads();
+        const int total = wcnt[0] + wcnt[1] + wcnt[2] + wcnt[3];
+        if (total == 0) continue;
+        int at = 0;
+        for (int w = 0; w < wave; w++) at += wcnt[w];
+        if (vis) list[at + __popcll(b & ((1ull << lane) - 1ull))] = c;
+        __syncthreads();
+        for (int l0 = 0; l0 < total; l0 += CA_TILE) {
+            const int nl = min(CA_TILE, total - l0);
+            if (l0) __syncthreads();
+            for (int i = tid; i < nl * D; i += 256) { const int cc = i / D, d = i % D; ksh[cc * DP + d] = kc[((int64_t) list[l0 + cc] * G + g) * D + d]; }
+            __syncthreads();
+            for (int i = tid; i < nl * hpg; i += 256) {
+                const int cc = i % nl, m = i / nl;
+                const float * kr = ksh + cc * DP, * qr = qsh + m * D;
+                float s = 0.0f;
+                for (int d = 0; d < D; d++) s = fmaf(qr[d], kr[d], s);
+                wsh[cc * hpg + m] = pm_sigmoid(s * scale + (hbias ? hbias[h0 + m] : 0.0f));
+            }
+            __syncthreads();
+#pragma unroll
+            for (int oi = 0; oi < CA_MAXOUT; oi++) {
+                const int o = oi * 256 + tid;
+                if (o < n_out) {
+                    const int m = o / V, vv = o % V;
+                    float a = acc[oi];
+                    for (int cc = 0; cc < nl; cc++) a = fmaf(wsh[cc * hpg + m], vc[((int64_t) list[l0 + cc] * G + g) * V + vv], a);
+                    acc[oi] = a;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int oi = 0; oi < CA_MAXOUT; oi++) {
+        const int o = oi * 256 + tid;
+        if (o < n_out) {
+            const int m = o / V;
+            float gt = gate ? gate[(int64_t) t * gs + h0 + m] : 1.0f;
+            if (gate && gate_act == PI_ACT_SIGMOID) gt = pm_sigmoid(gt);
+            out[(int64_t) t * os + (int64_t) h0 * V + o] = acc[oi] * gt;
+        }
+    }
+}
+
+extern "C" int pi_op_chunk_attention(const float * q, int64_t q_stride, const float * k_cache, const float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
+                                     const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, int chunk, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv,
+                                     float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
+    if (n_tok <= 0) return 0;
+    if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || vdim < 1 || chunk < 0) { pi_set_error("pi_op_chunk_attention: %d query heads over %d key / value heads, sizes %d / %d, chunk %d", heads, kv_heads, dim, vdim, chunk); return -1; }
+    const int hpg = heads / kv_heads;
+    const size_t lds = ((size_t) hpg * dim + (size_t) CA_TILE * (dim + 1) + (size_t) CA_TILE * hpg) * sizeof(float);
+    if (hpg * vdim > 256 * CA_MAXOUT || lds > 60 * 1024) { pi_set_error("pi_op_chunk_attention: %d query heads per key head of sizes %d / %d are beyond the kernel (LDS %zu bytes)", hpg, dim, vdim, lds); return -1; }
+    const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
+    const double visible = chunk > 0 ? std::min(acct, chunk) : acct;
+    PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention, dim3((unsigned) n_tok, (unsigned) kv_heads), dim3(256), lds,
+                 (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, chunk, heads, kv_heads, dim, vdim, n_kv, out, out_stride,
+                 dyn_dev, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// ---- short causal convolution over the tokens of each sequence ----------------------------------------------------------------------------------------------
+// rec[t]: state slot of token t's sequence (| 1 << 30 on the first token of a sequence that starts from nothing); a sequence's tokens are consecutive.
+// state: [slots][taps - 1][channels], the sequence's last inputs, oldest first.  grid (token, blocks of 256 channels)
+__global__ void __launch_bounds__(256) k_causal_conv(const float * __restrict__ x, int64_t xs, int channels, int taps, const float * __restrict__ w, const float * __restrict__ bias,
+                                                     const float * __restrict__ state, const int32_t * __restrict__ rec, int act, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= channels) return;
+    const int slot = rec[t] & ~PM_FRESH;
+    int d = 0, fresh = 0;                                             // d: tokens of this sequence in the pass before t (counted up to taps - 1)
+    while (d < taps - 1 && t - d - 1 >= 0 && (rec[t - d - 1] & ~PM_FRESH) == slot) d++;
+    if (d < taps - 1) fresh = (rec[t - d] & PM_FRESH) != 0;           // (t - d is then the sequence's first token of the pass)
+    float a = bias ? bias[c] : 0.0f;
+    for (int l = 0; l < taps; l++) {                                  // tap l weighs the input `taps - 1 - l` tokens back
+        const int back = taps - 1 - l;
+        float v;
+        if (back <= d) v = x[(int64_t) (t - back) * xs + c];
+        else v = fresh ? 0.0f : state[((int64_t) slot * (taps - 1) + (taps - 1 - (back - d))) * channels + c];
+        a = fmaf(w[(int64_t) c * taps + l], v, a);
+    }
+    if (act == PI_ACT_SILU) a = a / (1.0f + expf(-a));
+    out[(int64_t) t * os + c] = a;
+}
+// grid (token, blocks of 256 channels): only a sequence's last token of the pass works, it rewrites its slot's rows oldest first (a row only ever takes a later row's value)
+__global__ void __launch_bounds__(256) k_conv_state_update(const float * __restrict__ x, int64_t xs, int channels, int taps, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
+                                                           const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    const int slot = rec[t] & ~PM_FRESH;
+    if (t + 1 < n_tok && (rec[t + 1] & ~PM_FRESH) == slot) return;
+    if (c >= channels) return;
+    int len = 1, fresh = 0;                                           // tokens of the sequence in this pass, counted up to taps - 1
+    while (len < taps - 1 && t - len >= 0 && (rec[t - len] & ~PM_FRESH) == slot) len++;
+    if (len < taps - 1) fresh = (rec[t - len + 1] & PM_FRESH) != 0;
+    float * st = state + (int64_t) slot * (taps - 1) * channels + c;
+    for (int i = 0; i < taps - 1; i++) {
+        const int from = i + len;                                     // row of (old state, then the pass's tokens) that becomes row i
+        float v;
+        if (from < taps - 1) v = fresh ? 0.0f : st[(int64_t) from * channels];
+        else v = x[(int64_t) (t - len + 1 + from - (taps - 1)) * xs + c];
+        st[(int64_t) i * channels] = v;
+    }
+}
+
+extern "C" int pi_op_causal_conv(const float * x, int64_t x_stride, int channels, int taps, const float * w_dev, const float * bias_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int act,
+                                 float * out, int64_t out_stride, void * stream) {
+    if (n_tok <= 0 || channels <= 0) return 0;
+    if (taps < 1 || taps > 64) { pi_set_error("pi_op_causal_conv: %d taps (1..64)", taps); return -1; }
+    if (out == x) { pi_set_error("pi_op_causal_conv: the output may not overwrite the input (later tokens and the state read it)"); return -1; }
+    hipStream_t s = (hipStream_t) stream;
+    const dim3 grid((unsigned) n_tok, (unsigned) ((channels + 255) / 256));
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * n_tok * channels + 4.0 * channels * taps, k_causal_conv, grid, dim3(256), 0, s, x, x_stride, channels, taps, w_dev, bias_dev, state_dev, rec_dev, act, out, out_stride, pi_abort_word());
+    PI_CHECK_LAUNCH();
+    if (taps > 1) {
+        PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * (taps - 1) * channels, k_conv_state_update, grid, dim3(256), 0, s, x, x_stride, channels, taps, state_dev, rec_dev, n_tok, pi_abort_word());
+        PI_CHECK_LAUNCH();
+    }
+    return 0;
+}
+
+// ---- step sizes and decays of a selective recurrence ---------------------------------------------------------------------------------------------------------
+__global__ void k_ssd_steps(const float * __restrict__ raw, int64_t rs, const float * __restrict__ dt_bias, const float * __restrict__ a_log, int heads, int n_tok, float * __restrict__ dt,
+                            float * __restrict__ decay, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_tok * heads) return;
+    const int t = i / heads, h = i % heads;
+    const float z = raw[(int64_t) t * rs + h] + dt_bias[h];
+    const float sp = z > 20.0f ? z : log1pf(expf(z));                 // (beyond 20 the two agree to the last bit of fp32)
+    dt[i] = sp;
+    decay[i] = expf(-expf(a_log[h]) * sp);
+}
+extern "C" int pi_op_ssd_steps(const float * raw, int64_t raw_stride, const float * dt_bias_dev, const float * a_log_dev, int heads, int n_tok, float * dt_out, float * decay_out, void * stream) {
+    if (n_tok <= 0) return 0;
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 12.0 * n_tok * heads, k_ssd_steps, dim3((unsigned) ((n_tok * heads + 255) / 256)), dim3(256), 0, (hipStream_t) stream, raw, raw_stride, dt_bias_dev, a_log_dev, heads, n_tok,
+                 dt_out, decay_out, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// ---- gate, then RMS norm in equal parts -------------------------------------------------------------------------------------------------------------------
+// grid (token, part)
+__global__ void __launch_bounds__(256) k_gate_group_norm(const float * __restrict__ y, int64_t ys, const float * __restrict__ z, int64_t zs, const float * __restrict__ w, float eps, int n, int groups,
+                                                         float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    __shared__ float red[4];
+    const int t = blockIdx.x, part = n / groups, i0 = blockIdx.y * part;
+    const float * yr = y + (int64_t) t * ys + i0, * zr = z + (int64_t) t * zs + i0;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < part; i += 256) { const float g = zr[i], u = yr[i] * (g / (1.0f + expf(-g))); ss = fmaf(u, u, ss); }
+    ss = pm_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float) part + eps);
+    for (int i = threadIdx.x; i < part; i += 256) { const float g = zr[i], u = yr[i] * (g / (1.0f + expf(-g))); out[(int64_t) t * os + i0 + i] = u * inv * w[i0 + i]; }
+}
+extern "C" int pi_op_gate_group_norm(const float * y, int64_t y_stride, const float * z, int64_t z_stride, const float * w_dev, float eps, int n, int groups, int n_tok, float * out, int64_t out_stride, void * stream) {
+    if (n_tok <= 0 || n <= 0) return 0;
+    if (groups < 1 || n % groups) { pi_set_error("pi_op_gate_group_norm: %d values do not divide into %d equal parts", n, groups); return -1; }
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 16.0 * n * n_tok, k_gate_group_norm, dim3((unsigned) n_tok, (unsigned) groups), dim3(256), 0, (hipStream_t) stream, y, y_stride, z, z_stride, w_dev, eps, n, groups, out, out_stride,
+                 pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}

@@ -306,7 +306,7 @@ extern "C" enum llama_vocab_type llama_vocab_type(const struct llama_model * m) 
 extern "C" uint64_t llama_model_size(const struct llama_model * m) { return m->n_bytes; }
 extern "C" uint64_t llama_model_n_params(const struct llama_model * m) { return m->n_elements; }
 extern "C" int llama_model_desc(const struct llama_model * m, char * buf, size_t n) {
-    static const char * names[] = { "llama", "falcon", "baichuan", "starcoder", "refact", "bloom", "mpt", "stablelm", "persimmon", "fasovik" };
+    static const char * names[] = { "llama", "falcon", "baichuan", "starcoder", "refact", "bloom", "mpt", "stablelm", "persimmon", "fasovik", "vikarax" };
     return snprintf(buf, n, "%s %s", names[m->hparams.arch], m->name.c_str());
 }
 

@@ -150,3 +150,24 @@ def _declare(lib):
     lib.pi_op_latent_attention_max_cells.argtypes = [i32]
     lib.pi_op_moe_route.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp, vp, vp]
     lib.pi_op_moe_experts.argtypes = [vp, vp, i32, i32, vp, i64, vp, vp, i32, i32, i32, vp, vp, i64, vp]
+    lib.pi_op_moe_grouped_ok.argtypes = [vp, vp, i32, i32, i32, i32, i32, i32]
+    lib.pi_op_moe_grouped_index_ints.argtypes = [i32, i32, i32]; lib.pi_op_moe_grouped_index_ints.restype = sz
+    lib.pi_op_moe_experts_grouped.argtypes = [vp, vp, i32, i32, vp, i64, vp, vp, i32, i32, vp, vp, vp, vp, i64, vp]
+    # blocks with pre- and post-norms, the depth average, the parallel mixer's two branches, grouped routing and gated experts
+    lib.pi_op_layer_norm_mix.argtypes = [vp, i64, f32, vp, i64, f32, vp, vp, f32, i32, i32, vp, i64, vp, i64, vp]
+    lib.pi_op_depth_mix.argtypes = [vp, i64, i32, vp, i32, i32, vp, i64, vp]
+    lib.pi_op_softcap.argtypes = [vp, i64, f32, vp]
+    lib.pi_op_glu_mul.argtypes = [vp, i64, i32, i32, vp, i64, vp]
+    lib.pi_op_linear_attention_ex.argtypes = [vp, vp, vp, i64, i32, i32, i32, i32, vp, vp, vp, i64, vp, vp, vp, i32, i32, vp, sz, vp, i64, vp]
+    lib.pi_rotary_table_create.restype = vp
+    lib.pi_rotary_table_create.argtypes = [i32, i32, f32]
+    lib.pi_rotary_table_positions.argtypes = [vp]
+    lib.pi_rotary_table_free.argtypes = [vp]; lib.pi_rotary_table_free.restype = None
+    lib.pi_op_qkv_prepare.argtypes = [vp, vp, vp, i64, vp, vp, f32, i32, i32, i32, i32, vp, vp, i32, vp, i64, vp, vp, vp, vp, vp]
+    lib.pi_op_chunk_attention.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, i32, f32, i32, i32, i32, i32, i32, i32, i32, vp, i64, vp, vp]
+    lib.pi_op_causal_conv.argtypes = [vp, i64, i32, i32, vp, vp, vp, vp, i32, i32, vp, i64, vp]
+    lib.pi_op_ssd_steps.argtypes = [vp, i64, vp, vp, i32, i32, vp, vp, vp]
+    lib.pi_op_gate_group_norm.argtypes = [vp, i64, vp, i64, vp, f32, i32, i32, i32, vp, i64, vp]
+    lib.pi_op_moe_route_groups.argtypes = [vp, vp, i64, i32, i32, i32, i32, i32, vp, vp, vp]
+    lib.pi_op_moe_experts_act.argtypes = [vp, vp, i32, i32, i32, vp, i64, vp, vp, i32, i32, i32, vp, vp, i64, vp]
+    lib.pi_op_moe_experts_grouped_act.argtypes = [vp, vp, i32, i32, i32, vp, i64, vp, vp, i32, i32, vp, vp, vp, vp, i64, vp]

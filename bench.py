@@ -491,7 +491,12 @@ def main():
     ap.add_argument("--compare-hybrid", nargs="?", const="w1024,w2048,w4096", default=None, metavar="SIZES",
                     help="instead of the default workload: prefill / decode throughput and per-kernel roofline fractions of the Fasovik design at these layer sizes beside a Llama "
                          "model of equal size (pipeinfer_amd/tools/hybrid_bench.py); one JSON line per size")
+    ap.add_argument("--compare-parallel", nargs="?", const="w1024,w2048,w4096", default=None, metavar="SIZES",
+                    help="instead of the default workload: the same measurements for the Vikarax design (parallel mixer, gated experts) beside the Fasovik design at equal sizes; one JSON line per size")
     args = ap.parse_args()
+    if args.compare_parallel:
+        from pipeinfer_amd.tools import hybrid_bench
+        return hybrid_bench.main_parallel(args.compare_parallel.split(","), args.cache)
     if args.compare_hybrid:
         from pipeinfer_amd.tools import hybrid_bench
         return hybrid_bench.main(args.compare_hybrid.split(","), args.cache)

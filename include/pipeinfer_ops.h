@@ -219,6 +219,11 @@ PI_API int pi_op_moe_experts_grouped(const pi_weight * w_up, const pi_weight * w
 /* y = LayerNorm(ca * a + cb * b) * w + bias (b nullable: one input; the variance is the mean of squared deviations, eps inside the root); out = [residual +] y */
 PI_API int pi_op_layer_norm_mix(const float * a_dev, int64_t a_stride, float ca, const float * b_dev, int64_t b_stride, float cb, const float * w_dev, const float * bias_dev, float eps, int n, int n_tok,
                                 const float * residual_dev, int64_t residual_stride, float * out_dev, int64_t out_stride, void * stream);
+/* the end of a block in one launch: v = [residual +] LayerNorm(ca * a + cb * b) * w + bias -> out_a;  n_hist > 0: v = sum_(j < n_hist - 1) coef[j] * hist[j] + coef[n_hist - 1] * v -> out_mix
+ * (out_a must be the history's last entry, rows n floats apart);  w_next != NULL: LayerNorm(v) * w_next + bias_next -> out_next.  In place (out_a == residual, out_mix == residual) is allowed */
+PI_API int pi_op_norm_chain(const float * a_dev, int64_t a_stride, float ca, const float * b_dev, int64_t b_stride, float cb, const float * w_dev, const float * bias_dev, float eps, int n, int n_tok,
+                            const float * residual_dev, int64_t residual_stride, float * out_a_dev, int64_t out_a_stride, const float * hist_dev, int64_t hist_stride, int n_hist, const float * coef_dev,
+                            float * out_mix_dev, int64_t out_mix_stride, const float * w_next, const float * bias_next, float * out_next_dev, int64_t out_next_stride, void * stream);
 /* out[t] = sum_j coef[j] * hist[j][t], j = 0 .. n_hist - 1 in this order; hist: n_hist arrays of n_tok rows of n floats, hist_stride floats apart; coef_dev: fp32 [n_hist] */
 PI_API int pi_op_depth_mix(const float * hist_dev, int64_t hist_stride, int n_hist, const float * coef_dev, int n, int n_tok, float * out_dev, int64_t out_stride, void * stream);
 /* x <- cap * tanh(x / cap), in place */
@@ -240,20 +245,25 @@ PI_API void   pi_rotary_table_free(void * table);
 PI_API int pi_op_qkv_prepare(const float * q_dev, const float * k_dev, const float * v_dev, int64_t stride, const float * q_norm_w, const float * k_norm_w, float eps, int heads, int kv_heads, int dim, int vdim,
                              const void * rotary_table, const int32_t * pos_dev, int n_tok, float * q_out_dev, int64_t q_out_stride, float * k_cache_dev, float * v_cache_dev, int32_t * cell_pos_dev,
                              const int32_t * dyn_dev, void * stream);
-/* out[t][h] = gate[t][h] * sum over the cells c that token t sees of sigmoid(q[t][h] . K[c][h / (heads / kv_heads)] * scale + head_bias[h]) * V[c][..]: no soft-max, no normalisation.
+/* out[t][h] = out_mult * gate[t][h] * sum over the cells c that token t sees of sigmoid(q[t][h] . K[c][h / (heads / kv_heads)] * scale + head_bias[h]) * V[c][..]: no soft-max, no normalisation.
  * A cell is seen when its bit of the pass's mask is set AND (chunk > 0) its position is not below the start of the chunk of `chunk` positions that holds the token's position.
  * head_bias_dev, gate_dev nullable (0 and 1); gate_act: PI_ACT_SIGMOID when the gate values are still raw */
 PI_API int pi_op_chunk_attention(const float * q_dev, int64_t q_stride, const float * k_cache_dev, const float * v_cache_dev, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
-                                 const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, int chunk, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv,
+                                 const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int chunk, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv,
                                  float * out_dev, int64_t out_stride, const int32_t * dyn_dev, void * stream);
 /* out[t][c] = act(bias[c] + sum_l w[c][l] * input(t - (taps - 1 - l))[c]) over the tokens of each sequence (rec_dev as for pi_op_linear_attention); inputs from before the pass come from
  * state_dev [slots][taps - 1][channels] (oldest first; zeros for a sequence that starts), which then takes the sequence's last taps - 1 inputs.  w_dev: fp32 [channels][taps] */
 PI_API int pi_op_causal_conv(const float * x_dev, int64_t x_stride, int channels, int taps, const float * w_dev, const float * bias_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int act,
                              float * out_dev, int64_t out_stride, void * stream);
+/* pi_op_causal_conv and pi_op_ssd_steps together: ONE launch where the pass has at most 32 tokens and the convolution at most 8 taps (a sequence's tokens are then walked by one
+ * thread per channel, which also leaves the new state), the separate launches otherwise */
+PI_API int pi_op_causal_conv_steps(const float * x_dev, int64_t x_stride, int channels, int taps, const float * w_dev, const float * bias_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int act,
+                                   float * out_dev, int64_t out_stride, const float * raw_dev, int64_t raw_stride, const float * dt_bias_dev, const float * a_log_dev, int heads, float * dt_out_dev,
+                                   float * decay_out_dev, void * stream);
 /* dt[t][h] = softplus(raw[t][h] + dt_bias[h]); decay[t][h] = exp(-exp(a_log[h]) * dt[t][h]); outputs [n_tok][heads] */
 PI_API int pi_op_ssd_steps(const float * raw_dev, int64_t raw_stride, const float * dt_bias_dev, const float * a_log_dev, int heads, int n_tok, float * dt_out_dev, float * decay_out_dev, void * stream);
-/* u = y * silu(z); out = u / rms(u over each of `groups` equal parts) * w */
-PI_API int pi_op_gate_group_norm(const float * y_dev, int64_t y_stride, const float * z_dev, int64_t z_stride, const float * w_dev, float eps, int n, int groups, int n_tok, float * out_dev, int64_t out_stride, void * stream);
+/* u = y * silu(z); out = u / rms(u over each of `groups` equal parts) * w * mult */
+PI_API int pi_op_gate_group_norm(const float * y_dev, int64_t y_stride, const float * z_dev, int64_t z_stride, const float * w_dev, float eps, float mult, int n, int groups, int n_tok, float * out_dev, int64_t out_stride, void * stream);
 /* router with sigmoid scores and a choice limited to groups: the outputs form n_groups equal groups of neighbours, a group's score is the sum of its two largest scores, only outputs of the
  * `keep` best groups can be chosen; the `top` largest scores among them win and are the weights (not renormalised) */
 PI_API int pi_op_moe_route_groups(const pi_weight * router, const float * x_dev, int64_t x_stride, int n_tok, int top, int n_groups, int keep, int exact, int32_t * sel_dev, float * selw_dev, void * stream);

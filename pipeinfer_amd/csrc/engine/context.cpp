@@ -293,36 +293,37 @@ static bool mul_mat_grouped(int n, const pi_weight * const * ws, const void * co
 //
 // Blocks with norms before AND after every sublayer (hp.pre_post_norm) and a learned average over depth (hp.depth_average):
 //   h = LN1(x); x += LN1b(a * attention_branch(h) + b * recurrence_branch(h));  h = LN2(x); x += LN2b(ff(h));  X_(i+1) = x;  x = sum_j c_ij X_j
-// Kernel sequence of a parallel mixer: norm -> ONE projection [q | k | v | gate | z | x | B | C | dt] -> (q/k norm + rotation, v norm, cache store) -> chunked sigmoid attention ->
-// W_o;  convolution (+ its state) -> step sizes -> recurrence -> gate + grouped norm -> W_o';  post-norm of the weighted sum + residual.  The stream after every layer is kept
-// in ctx->hist for the depth average; the block's last norm writes X_(i+1) straight into it.
+// Kernel sequence of a parallel mixer: ONE projection [q | k | v | gate | z | x | B | C | dt] -> (q/k norm + rotation, v norm, cache store) -> chunked sigmoid attention;
+// convolution (+ its state, + step sizes) -> recurrence -> gate + grouped norm;  ONE output projection [W_o | W_o'] over both branches' outputs (each already times its factor).
+// Every norm, residual sum and the depth average between two matrix products is one row kernel (pi_op_norm_chain); the stream after every layer is kept in ctx->hist.
 static bool forward_parallel_mixer(llama_context * ctx, const pi_hybrid_layer & H, const pi_hybrid_weights & W, size_t il, const float * N, int n_tok, int n_kv) {
     const pi_hparams & hp = ctx->model->hparams;
     hipStream_t s = ctx->stream;
     const int width = hp.n_embd, ex = ctx->exact, nb = ctx->n_batch;
     const float eps = hp.f_norm_eps;
     const pi_gate_attention & A = H.left; const pi_ssd & R = H.right;
-    const int64_t pw = H.in_rows(), hd = (int64_t) A.heads * A.dim, hv = (int64_t) A.heads * A.vdim, gd = (int64_t) A.kv_heads * A.dim, gv = (int64_t) A.kv_heads * A.vdim;
-    float * P = ctx->h_in, * Q = ctx->h_att, * O = Q + (size_t) nb * hd, * C = O + (size_t) nb * hv, * S = C + (size_t) nb * R.channels();
+    const int inner = R.inner(), gn = R.groups * R.state;
+    const int64_t pw = H.in_rows(), hd = (int64_t) A.heads * A.dim, hv = (int64_t) A.heads * A.vdim, gd = (int64_t) A.kv_heads * A.dim, gv = (int64_t) A.kv_heads * A.vdim, ow = hv + inner;
+    // scratch: rotated queries | both branches' outputs side by side (the input rows of the ONE output projection [W_o | W_o']) | the convolution's output
+    float * P = ctx->h_in, * Q = ctx->h_att, * O = Q + (size_t) nb * hd, * S = O + hv, * C = O + (size_t) nb * ow;
     float * kc = ctx->lat_cache + ctx->lat_off[il], * vc = kc + (size_t) ctx->n_ctx * gd;
     float * ssm = ctx->rec_state + ctx->rec_off[il], * conv_state = ssm + (size_t) ctx->slots->size() * R.heads * R.state * R.vdim;
     OP_OK(pi_op_dense(W.w_in, N, width, n_tok, P, pw, PI_ACT_NONE, pw, PI_ACT_NONE, ex, s));
-    // attention branch
+    // attention branch (its output already carries the branch's factor)
     OP_OK(pi_op_qkv_prepare(P, P + hd, P + hd + gd, pw, W.q_norm, W.k_norm, eps, A.heads, A.kv_heads, A.dim, A.vdim, W.rotary, ctx->pos_dev, n_tok, Q, hd, kc, vc, ctx->cell_pos, ctx->dyn_dev, s));
-    OP_OK(pi_op_chunk_attention(Q, hd, kc, vc, ctx->cell_pos, ctx->mask_dev, ctx->pos_dev, W.head_bias, P + hd + gd + gv, pw, PI_ACT_SIGMOID, A.scale, A.chunk, A.heads, A.kv_heads, A.dim, A.vdim, n_tok, n_kv, O, hv, ctx->dyn_dev, s));
-    trace(ctx, "att", (int) il, O, hv, n_tok);
-    OP_OK(pi_op_dense(W.w_o, O, hv, n_tok, ctx->h_out, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+    OP_OK(pi_op_chunk_attention(Q, hd, kc, vc, ctx->cell_pos, ctx->mask_dev, ctx->pos_dev, W.head_bias, P + hd + gd + gv, pw, PI_ACT_SIGMOID, A.scale, H.left_scale, A.chunk, A.heads, A.kv_heads, A.dim, A.vdim, n_tok, n_kv,
+                                O, ow, ctx->dyn_dev, s));
+    trace(ctx, "att", (int) il, O, hv, n_tok, ow);
     // recurrence branch
     const float * R0 = P + A.in_rows();                                   // z | x B C | dt
-    const int inner = R.inner(), gn = R.groups * R.state;
     float * dt = ctx->ssd_dt, * decay = dt + (size_t) nb * R.heads;
-    OP_OK(pi_op_causal_conv(R0 + inner, pw, R.channels(), R.conv, W.conv_w, W.conv_b, conv_state, ctx->rec_dev, n_tok, PI_ACT_SILU, C, R.channels(), s));
-    OP_OK(pi_op_ssd_steps(R0 + inner + R.channels(), pw, W.dt_bias, W.a_log, R.heads, n_tok, dt, decay, s));
+    OP_OK(pi_op_causal_conv_steps(R0 + inner, pw, R.channels(), R.conv, W.conv_w, W.conv_b, conv_state, ctx->rec_dev, n_tok, PI_ACT_SILU, C, R.channels(),
+                                  R0 + inner + R.channels(), pw, W.dt_bias, W.a_log, R.heads, dt, decay, s));
     OP_OK(pi_op_linear_attention_ex(C + inner + gn, C + inner, C, R.channels(), R.heads, R.groups, R.state, R.vdim, nullptr, decay, dt, R.heads, W.skip, ssm, ctx->rec_dev, n_tok, ctx->slots->size(),
-                                    ctx->rec_scratch, ctx->rec_scratch_floats, S, inner, s));
-    OP_OK(pi_op_gate_group_norm(S, inner, R0, pw, W.mix_norm, eps, inner, R.norm_groups, n_tok, S, inner, s));
-    trace(ctx, "ssd", (int) il, S, inner, n_tok);
-    OP_OK(pi_op_dense(W.w_o2, S, inner, n_tok, ctx->h_out2, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+                                    ctx->rec_scratch, ctx->rec_scratch_floats, S, ow, s));
+    OP_OK(pi_op_gate_group_norm(S, ow, R0, pw, W.mix_norm, eps, H.right_scale, inner, R.norm_groups, n_tok, S, ow, s));
+    trace(ctx, "ssd", (int) il, S, inner, n_tok, ow);
+    OP_OK(pi_op_dense(W.w_o, O, ow, n_tok, ctx->h_out, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));          // a * W_o att + b * W_o' rec
     return true;
 }
 
@@ -333,25 +334,31 @@ static bool forward_pre_post_blocks(llama_context * ctx, int n_tok, int n_kv) {
     const int width = hp.n_embd, ex = ctx->exact, nb = ctx->n_batch;
     const float eps = hp.f_norm_eps;
     const size_t hs = (size_t) nb * width;
+    const size_t n_layer = hp.hybrid.size();
     float * P = ctx->h_in, * N = ctx->nx, * Y = ctx->h_out, * Y2 = ctx->h_out2;
     float * x = hp.depth_average ? ctx->hist : ctx->x;                    // the embedding output is X_0
     OP_OK(pi_op_embed(m->tok_embd, ctx->tokens_dev, n_tok, hp.embed_scale, x, s));
-    for (size_t il = 0; il < hp.hybrid.size(); il++) {
+    OP_OK(pi_op_layer_norm_mix(x, width, 1.0f, nullptr, 0, 0.0f, m->hweights[(size_t) hp.hybrid[0].weights].norm1, m->hweights[(size_t) hp.hybrid[0].weights].norm1_b, eps, width, n_tok, nullptr, 0, N, width, s));
+    for (size_t il = 0; il < n_layer; il++) {
         const pi_hybrid_layer & H = hp.hybrid[il];
         const pi_hybrid_weights & W = m->hweights[(size_t) H.weights];
-        float * X_next = hp.depth_average ? ctx->hist + (il + 1) * hs : ctx->x;     // where the block's result goes
-        float * after_mixer = H.has_mlp ? ctx->x : X_next;
-        OP_OK(pi_op_layer_norm_mix(x, width, 1.0f, nullptr, 0, 0.0f, W.norm1, W.norm1_b, eps, width, n_tok, nullptr, 0, N, width, s));
+        // a block ends in ONE row kernel: post-norm + residual -> X_(i+1) (into the history), the depth average -> x, the pre-norm of what comes next (the next layer, or the output) -> N
+        const float * next_w = il + 1 < n_layer ? m->hweights[(size_t) hp.hybrid[il + 1].weights].norm1 : m->output_norm, * next_b = il + 1 < n_layer ? m->hweights[(size_t) hp.hybrid[il + 1].weights].norm1_b : m->output_norm_b;
+        auto block_end = [&](const float * a, const float * b2, const float * w, const float * wb, const float * res) {
+            if (hp.depth_average) return pi_op_norm_chain(a, width, 1.0f, b2, width, 1.0f, w, wb, eps, width, n_tok, res, width, ctx->hist + (il + 1) * hs, width, ctx->hist, (int64_t) hs, (int) il + 2, W.depth, ctx->x, width,
+                                                          next_w, next_b, N, width, s);
+            return pi_op_norm_chain(a, width, 1.0f, b2, width, 1.0f, w, wb, eps, width, n_tok, res, width, ctx->x, width, nullptr, 0, 0, nullptr, nullptr, 0, next_w, next_b, N, width, s);
+        };
         if (H.mixer != PI_MIXER_PARALLEL) { ctx->last_error = "blocks with norms on both sides of a sublayer are built for the parallel mixer"; return false; }
         if (!forward_parallel_mixer(ctx, H, W, il, N, n_tok, n_kv)) return false;
-        OP_OK(pi_op_layer_norm_mix(Y, width, H.left_scale, Y2, width, H.right_scale, W.post1, W.post1_b, eps, width, n_tok, x, width, after_mixer, width, s));
-        if (H.has_mlp) {
-            x = after_mixer;
-            OP_OK(pi_op_layer_norm_mix(x, width, 1.0f, nullptr, 0, 0.0f, W.norm2, W.norm2_b, eps, width, n_tok, nullptr, 0, N, width, s));
+        if (!H.has_mlp) OP_OK(block_end(Y, nullptr, W.post1, W.post1_b, x));
+        else {
+            OP_OK(pi_op_norm_chain(Y, width, 1.0f, nullptr, 0, 0.0f, W.post1, W.post1_b, eps, width, n_tok, x, width, ctx->x, width, nullptr, 0, 0, nullptr, nullptr, 0, W.norm2, W.norm2_b, N, width, s));   // + the feed-forward's pre-norm
+            x = ctx->x;
             if (H.mlp == PI_MLP_DENSE_RELU_SQR) {
                 OP_OK(pi_op_dense(W.ff_up, N, width, n_tok, P, H.ff, PI_ACT_RELU_SQR, H.ff, PI_ACT_RELU_SQR, ex, s));
                 OP_OK(pi_op_dense(W.ff_down, P, H.ff, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
-                OP_OK(pi_op_layer_norm_mix(Y, width, 1.0f, nullptr, 0, 0.0f, W.post2, W.post2_b, eps, width, n_tok, x, width, X_next, width, s));
+                OP_OK(block_end(Y, nullptr, W.post2, W.post2_b, x));
             } else {
                 OP_OK(pi_op_moe_route_groups(W.router, N, width, n_tok, H.top, H.route_groups, H.route_keep, ex, ctx->moe_sel, ctx->moe_w, s));
                 if (pi_op_moe_grouped_ok(W.e_up, W.e_down, H.n_expert, H.ff, 1, n_tok, H.top, ex))                                                // prompts: by expert, on the matrix cores
@@ -365,14 +372,12 @@ static bool forward_pre_post_blocks(llama_context * ctx, int n_tok, int n_kv) {
                     OP_OK(pi_op_glu_mul(P, 2 * sf, sf, n_tok, G, sf, s));
                     OP_OK(pi_op_dense(W.ff_down, G, sf, n_tok, Y2, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
                 }
-                OP_OK(pi_op_layer_norm_mix(Y, width, 1.0f, H.shared_ff > 0 ? Y2 : nullptr, width, 1.0f, W.post2, W.post2_b, eps, width, n_tok, x, width, X_next, width, s));
+                OP_OK(block_end(Y, H.shared_ff > 0 ? Y2 : nullptr, W.post2, W.post2_b, x));
             }
         }
-        x = X_next;
-        if (hp.depth_average) { OP_OK(pi_op_depth_mix(ctx->hist, (int64_t) hs, (int) il + 2, W.depth, width, n_tok, ctx->x, width, s)); x = ctx->x; }
+        x = ctx->x;
         trace(ctx, "lout", (int) il, x, width, n_tok);
     }
-    OP_OK(pi_op_layer_norm_mix(x, width, 1.0f, nullptr, 0, 0.0f, m->output_norm, m->output_norm_b, eps, width, n_tok, nullptr, 0, N, width, s));
     OP_OK(pi_op_dense(hp.own_head ? m->output : m->tok_embd, N, width, n_tok, ctx->logits_dev, hp.n_vocab, PI_ACT_NONE, hp.n_vocab, PI_ACT_NONE, ex, s));
     if (hp.logit_softcap > 0.0f) OP_OK(pi_op_softcap(ctx->logits_dev, (int64_t) n_tok * hp.n_vocab, hp.logit_softcap, s));
     OP_OK(pi_op_topk(ctx->logits_dev, hp.n_vocab, n_tok, 8, ctx->topk_ids_dev, ctx->topk_vals_dev, ctx->topk_sum_dev, ctx->topk_scratch_dev, s));

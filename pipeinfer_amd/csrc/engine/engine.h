@@ -80,8 +80,8 @@ struct pi_hybrid_weights {                            // the tensors of a layer 
     pi_weight * w_in = nullptr;                       // latent attention: [q | dkv], lightning: [q | k | v | g] (projections of the same input, one matrix)
     pi_weight * w_uk = nullptr, * w_uv = nullptr, * w_o = nullptr, * router = nullptr, * e_up = nullptr, * e_down = nullptr;
     float * norm1 = nullptr, * norm2 = nullptr, * mix_norm = nullptr, * sink = nullptr, * decay = nullptr, * correction = nullptr;
-    // parallel mixer: w_in = [q | k | v | gate | z | x | B | C | dt], w_o = the attention branch's output projection, w_o2 = the recurrence's; dense / shared feed-forward: [up] or [gate | up], down
-    pi_weight * w_o2 = nullptr, * ff_up = nullptr, * ff_down = nullptr;
+    // parallel mixer: w_in = rows [q | k | v | gate | z | x | B | C | dt], w_o = COLUMNS [attention branch's W_o | recurrence's W_o]; dense / shared feed-forward: [up] or [gate | up], down
+    pi_weight * ff_up = nullptr, * ff_down = nullptr;
     float * norm1_b = nullptr, * norm2_b = nullptr, * post1 = nullptr, * post1_b = nullptr, * post2 = nullptr, * post2_b = nullptr, * depth = nullptr;      // biases of the pre-norms, the post-norms, the depth average's factors
     float * q_norm = nullptr, * k_norm = nullptr, * head_bias = nullptr, * conv_w = nullptr, * conv_b = nullptr, * dt_bias = nullptr, * a_log = nullptr, * skip = nullptr;
     void * rotary = nullptr;                          // pi_rotary_table of the layer's (dims, base)

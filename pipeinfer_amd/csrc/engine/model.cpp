@@ -40,7 +40,7 @@ llama_model::~llama_model() {
         pi_weight_free(l.ffn_gate); pi_weight_free(l.ffn_down); pi_weight_free(l.ffn_up);
     }
     for (auto & w : hweights) { pi_weight_free(w.w_in); pi_weight_free(w.w_uk); pi_weight_free(w.w_uv); pi_weight_free(w.w_o); pi_weight_free(w.router); pi_weight_free(w.e_up); pi_weight_free(w.e_down);
-                                pi_weight_free(w.w_o2); pi_weight_free(w.ff_up); pi_weight_free(w.ff_down); if (w.rotary) pi_rotary_table_free(w.rotary); }
+                                pi_weight_free(w.ff_up); pi_weight_free(w.ff_down); if (w.rotary) pi_rotary_table_free(w.rotary); }
     for (void * t : retired_tables) pi_rotary_table_free(t);
     pi_weight_free(tok_embd); pi_weight_free(output); pi_weight_free(pos_embd);
     for (void * p : f32_allocs) pi_free(p);

@@ -57,6 +57,24 @@ struct loader {
         m.matrices.push_back({ w, nullptr, -1 });
         return w;
     }
+    // columns of several [rows][k_i] tensors side by side as one bfloat16 matrix [rows][sum k_i] (projections whose outputs are summed: one product over the concatenated inputs)
+    pi_weight * matrix_cols(const std::vector<std::pair<std::string, int64_t>> & parts, int64_t rows) {
+        int64_t k = 0;
+        for (const auto & p : parts) k += p.second;
+        std::vector<uint16_t> host((size_t) (rows * k));
+        int64_t at = 0;
+        for (const auto & p : parts) {
+            const pi::st_tensor * t = get(p.first, { rows, p.second });
+            if (!t) return nullptr;
+            for (int64_t r = 0; r < rows; r++) memcpy(host.data() + r * k + at, (const uint16_t *) t->data + r * p.second, (size_t) p.second * 2);
+            at += p.second;
+        }
+        pi_weight * w = pi_weight_upload(PI_BF16, k, rows, host.data(), nullptr);
+        if (!w) { err = "upload of " + parts[0].first + " failed: " + pi_last_error(); return nullptr; }
+        m.hbm_bytes += pi_weight_nbytes(w);
+        m.matrices.push_back({ w, nullptr, -1 });
+        return w;
+    }
     float * vector_f32(const std::vector<float> & v) {
         float * d = (float *) pi_malloc(std::max<size_t>(v.size(), 1) * 4);
         if (!d || (!v.empty() && (pi_memcpy_h2d(d, v.data(), v.size() * 4, nullptr) || pi_stream_sync(nullptr)))) { err = std::string("upload of a vector failed: ") + pi_last_error(); return nullptr; }
@@ -179,7 +197,7 @@ bool llama_model::ensure_loaded_hybrid(int n_positions, std::string & err) {
             if (hp.depth_average && !(W.depth = L.vector(p + "dwa", (int64_t) i + 2))) return false;
             if (!(W.w_in = L.matrix({ { l + "q", (int64_t) A.heads * A.dim }, { l + "k", (int64_t) A.kv_heads * A.dim }, { l + "v", (int64_t) A.kv_heads * A.vdim }, { l + "g", A.heads }, { r + "in", R.in_rows() } }, width))) return false;
             if (!(W.q_norm = L.vector(l + "q.norm", A.dim)) || !(W.k_norm = L.vector(l + "k.norm", A.dim)) || !(W.head_bias = L.vector(l + "pb", A.heads))) return false;
-            if (!(W.w_o = L.matrix({ { l + "o", width } }, (int64_t) A.heads * A.vdim)) || !(W.w_o2 = L.matrix({ { r + "o", width } }, R.inner()))) return false;
+            if (!(W.w_o = L.matrix_cols({ { l + "o", (int64_t) A.heads * A.vdim }, { r + "o", R.inner() } }, width))) return false;      // [W_o | W_o']: both branches' outputs enter one product
             if (!(W.conv_w = L.vector2(r + "conv", R.channels(), R.conv)) || !(W.conv_b = L.vector(r + "conv.b", R.channels()))) return false;
             if (!(W.dt_bias = L.vector(r + "dt_bias", R.heads)) || !(W.a_log = L.vector(r + "A_log", R.heads)) || !(W.skip = L.vector(r + "D", R.heads)) || !(W.mix_norm = L.vector(r + "norm", R.inner()))) return false;
             if (!(W.rotary = pi_rotary_table_create(std::max(n_positions, 32), A.rot_dims, A.rot_base))) { err = std::string("rotation table: ") + pi_last_error(); return false; }

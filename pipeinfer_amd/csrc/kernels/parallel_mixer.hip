@@ -7,8 +7,9 @@
 //   k_chunk_attention    out[t][h] = gate[t][h] * sum over visible cells c of sigmoid(q . K[c] * scale + bias[h]) V[c];  visible = the pass's mask bit AND position(c) >= start of t's chunk
 //   k_causal_conv        per channel: act(bias + sum_l w[l] * input(t - taps + 1 + l)), inputs before the pass come from the sequence's conv state (zeros for a fresh one)
 //   k_conv_state_update  the sequence's last taps - 1 inputs, for the next pass
+//   k_causal_conv_walk   both of the above and k_ssd_steps in one launch for passes of at most 32 tokens
 //   k_ssd_steps          dt = softplus(raw + bias), a = exp(-exp(A_log) * dt)
-//   k_gate_group_norm    u = y * silu(z); each of `groups` equal parts of u divided by its root mean square; * w
+//   k_gate_group_norm    u = y * silu(z); each of `groups` equal parts of u divided by its root mean square; * w * mult
 #include "ops_common.h"
 #include "kernel_timing.h"
 
@@ -106,18 +107,18 @@ extern "C" int pi_op_qkv_prepare(const float * q, const float * k, const float *
 // grid (token, key / value head): the workgroup serves the `hpg` query heads of its key head.  The cells are walked 256 at a time; the visible ones of a block are compacted
 // in cell order (so that the sum has one order whatever the launch), their key rows staged in LDS 64 at a time.  Scores: thread (cell, query head); output: thread (query
 // head, value column), value rows read from the cache along the columns.
-#define CA_TILE 64
+#define CA_TILE 64                                // key rows staged at a time (fewer when a row is long: ca_tile)
 #define CA_MAXOUT 16                              // outputs (query head, value column) a thread accumulates: hpg * vdim <= 256 * CA_MAXOUT
 __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * __restrict__ kc, const float * __restrict__ vc, const int32_t * __restrict__ cell_pos,
                                                          const uint32_t * __restrict__ mask, const int32_t * __restrict__ pos, const float * __restrict__ hbias, const float * __restrict__ gate, int64_t gs, int gate_act,
-                                                         float scale, int chunk, int H, int G, int D, int V, int n_kv_arg, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
+                                                         float scale, float out_mult, int chunk, int H, int G, int D, int V, int n_kv_arg, int tile, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
                                                          const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
-    extern __shared__ float lds[];                // q [hpg][D] | key tile [CA_TILE][D + 1] | weights [CA_TILE][hpg]
+    extern __shared__ float lds[];                // q [hpg][D] | key tile [tile][D + 1] | weights [tile][hpg]
     __shared__ int list[256], wcnt[4];
     const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hpg = H / G, h0 = g * hpg, DP = D + 1;
-    float * qsh = lds, * ksh = qsh + hpg * D, * wsh = ksh + CA_TILE * DP;
+    float * qsh = lds, * ksh = qsh + hpg * D, * wsh = ksh + tile * DP;
     const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg);
     const int words = (n_kv_arg + 31) / 32;
     const uint32_t * mrow = mask + (int64_t) t * words;
@@ -142,8 +143,8 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
         for (int w = 0; w < wave; w++) at += wcnt[w];
         if (vis) list[at + __popcll(b & ((1ull << lane) - 1ull))] = c;
         __syncthreads();
-        for (int l0 = 0; l0 < total; l0 += CA_TILE) {
-            const int nl = min(CA_TILE, total - l0);
+        for (int l0 = 0; l0 < total; l0 += tile) {
+            const int nl = min(tile, total - l0);
             if (l0) __syncthreads();
             for (int i = tid; i < nl * D; i += 256) { const int cc = i / D, d = i % D; ksh[cc * DP + d] = kc[((int64_t) list[l0 + cc] * G + g) * D + d]; }
             __syncthreads();
@@ -174,23 +175,26 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
             const int m = o / V;
             float gt = gate ? gate[(int64_t) t * gs + h0 + m] : 1.0f;
             if (gate && gate_act == PI_ACT_SIGMOID) gt = pm_sigmoid(gt);
-            out[(int64_t) t * os + (int64_t) h0 * V + o] = acc[oi] * gt;
+            out[(int64_t) t * os + (int64_t) h0 * V + o] = acc[oi] * gt * out_mult;
         }
     }
 }
 
 extern "C" int pi_op_chunk_attention(const float * q, int64_t q_stride, const float * k_cache, const float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
-                                     const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, int chunk, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv,
+                                     const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int chunk, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv,
                                      float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
     if (n_tok <= 0) return 0;
     if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || vdim < 1 || chunk < 0) { pi_set_error("pi_op_chunk_attention: %d query heads over %d key / value heads, sizes %d / %d, chunk %d", heads, kv_heads, dim, vdim, chunk); return -1; }
     const int hpg = heads / kv_heads;
-    const size_t lds = ((size_t) hpg * dim + (size_t) CA_TILE * (dim + 1) + (size_t) CA_TILE * hpg) * sizeof(float);
+    int tile = CA_TILE;
+    auto lds_of = [&](int tl) { return ((size_t) hpg * dim + (size_t) tl * (dim + 1) + (size_t) tl * hpg) * sizeof(float); };
+    while (tile > 4 && lds_of(tile) > 60 * 1024) tile >>= 1;
+    const size_t lds = lds_of(tile);
     if (hpg * vdim > 256 * CA_MAXOUT || lds > 60 * 1024) { pi_set_error("pi_op_chunk_attention: %d query heads per key head of sizes %d / %d are beyond the kernel (LDS %zu bytes)", hpg, dim, vdim, lds); return -1; }
     const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
     const double visible = chunk > 0 ? std::min(acct, chunk) : acct;
     PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention, dim3((unsigned) n_tok, (unsigned) kv_heads), dim3(256), lds,
-                 (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, chunk, heads, kv_heads, dim, vdim, n_kv, out, out_stride,
+                 (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, chunk, heads, kv_heads, dim, vdim, n_kv, tile, out, out_stride,
                  dyn_dev, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
 }
@@ -255,6 +259,68 @@ extern "C" int pi_op_causal_conv(const float * x, int64_t x_stride, int channels
     return 0;
 }
 
+// Short passes (decoding, small portions) in ONE launch: the thread of a sequence's FIRST token of the pass walks that sequence's tokens for its channel with the window in
+// registers and leaves the new state, so no other thread reads what it writes; one extra row of blocks computes the recurrence's step sizes and decays meanwhile.
+#define CV_MAXTAPS 8
+__global__ void __launch_bounds__(256) k_causal_conv_walk(const float * __restrict__ x, int64_t xs, int channels, int taps, const float * __restrict__ w, const float * __restrict__ bias,
+                                                          float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, int act, float * __restrict__ out, int64_t os, int cblocks,
+                                                          const float * __restrict__ raw, int64_t raws, const float * __restrict__ dt_bias, const float * __restrict__ a_log, int heads,
+                                                          float * __restrict__ dt, float * __restrict__ decay, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x;
+    if ((int) blockIdx.y == cblocks) {                                // step sizes and decays of token t
+        for (int h = threadIdx.x; h < heads; h += 256) {
+            const float z = raw[(int64_t) t * raws + h] + dt_bias[h];
+            const float sp = z > 20.0f ? z : log1pf(expf(z));
+            dt[(int64_t) t * heads + h] = sp;
+            decay[(int64_t) t * heads + h] = expf(-expf(a_log[h]) * sp);
+        }
+        return;
+    }
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    const int word = rec[t], slot = word & ~PM_FRESH;
+    if (c >= channels || (t > 0 && (rec[t - 1] & ~PM_FRESH) == slot)) return;
+    float win[CV_MAXTAPS - 1], wt[CV_MAXTAPS];                         // right-aligned (the last entries are the most recent input / the current token's tap): every register index is static
+    const int off = CV_MAXTAPS - taps;
+    float * st = state + (int64_t) slot * (taps - 1) * channels + c;
+#pragma unroll
+    for (int l = 0; l < CV_MAXTAPS - 1; l++) win[l] = l >= off && !(word & PM_FRESH) ? st[(int64_t) (l - off) * channels] : 0.0f;
+#pragma unroll
+    for (int l = 0; l < CV_MAXTAPS; l++) wt[l] = l >= off ? w[(int64_t) c * taps + (l - off)] : 0.0f;
+    const float b0 = bias ? bias[c] : 0.0f;
+    for (int tt = t; tt < n_tok && (rec[tt] & ~PM_FRESH) == slot; tt++) {
+        const float v = x[(int64_t) tt * xs + c];
+        float a = b0;
+#pragma unroll
+        for (int l = 0; l < CV_MAXTAPS - 1; l++) a = fmaf(wt[l], win[l], a);       // (entries left of the window carry zero weights)
+        a = fmaf(wt[CV_MAXTAPS - 1], v, a);
+#pragma unroll
+        for (int l = 0; l < CV_MAXTAPS - 2; l++) win[l] = win[l + 1];
+        win[CV_MAXTAPS - 2] = v;
+        if (act == PI_ACT_SILU) a = a / (1.0f + expf(-a));
+        out[(int64_t) tt * os + c] = a;
+    }
+#pragma unroll
+    for (int l = 0; l < CV_MAXTAPS - 1; l++) if (l >= off) st[(int64_t) (l - off) * channels] = win[l];
+}
+#define CV_WALK_MAX_TOKENS 32
+// the convolution and, in the same launch where the pass is short, the step sizes / decays of the recurrence it feeds (raw_dev .. decay_out as for pi_op_ssd_steps)
+extern "C" int pi_op_causal_conv_steps(const float * x, int64_t x_stride, int channels, int taps, const float * w_dev, const float * bias_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int act,
+                                       float * out, int64_t out_stride, const float * raw, int64_t raw_stride, const float * dt_bias_dev, const float * a_log_dev, int heads, float * dt_out, float * decay_out,
+                                       void * stream) {
+    if (n_tok <= 0 || channels <= 0) return 0;
+    if (taps < 1 || taps > 64) { pi_set_error("pi_op_causal_conv: %d taps (1..64)", taps); return -1; }
+    if (n_tok > CV_WALK_MAX_TOKENS || taps > CV_MAXTAPS) {
+        if (pi_op_causal_conv(x, x_stride, channels, taps, w_dev, bias_dev, state_dev, rec_dev, n_tok, act, out, out_stride, stream) != 0) return -1;
+        return pi_op_ssd_steps(raw, raw_stride, dt_bias_dev, a_log_dev, heads, n_tok, dt_out, decay_out, stream);
+    }
+    if (out == x) { pi_set_error("pi_op_causal_conv: the output may not overwrite the input"); return -1; }
+    const int cblocks = (channels + 255) / 256;
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * n_tok * channels + 4.0 * channels * (2 * taps - 1) + 12.0 * n_tok * heads, k_causal_conv_walk, dim3((unsigned) n_tok, (unsigned) (cblocks + 1)), dim3(256), 0, (hipStream_t) stream,
+                 x, x_stride, channels, taps, w_dev, bias_dev, state_dev, rec_dev, n_tok, act, out, out_stride, cblocks, raw, raw_stride, dt_bias_dev, a_log_dev, heads, dt_out, decay_out, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
 // ---- step sizes and decays of a selective recurrence ---------------------------------------------------------------------------------------------------------
 __global__ void k_ssd_steps(const float * __restrict__ raw, int64_t rs, const float * __restrict__ dt_bias, const float * __restrict__ a_log, int heads, int n_tok, float * __restrict__ dt,
                             float * __restrict__ decay, const int32_t * __restrict__ abort_w) {
@@ -276,7 +342,7 @@ extern "C" int pi_op_ssd_steps(const float * raw, int64_t raw_stride, const floa
 
 // ---- gate, then RMS norm in equal parts -------------------------------------------------------------------------------------------------------------------
 // grid (token, part)
-__global__ void __launch_bounds__(256) k_gate_group_norm(const float * __restrict__ y, int64_t ys, const float * __restrict__ z, int64_t zs, const float * __restrict__ w, float eps, int n, int groups,
+__global__ void __launch_bounds__(256) k_gate_group_norm(const float * __restrict__ y, int64_t ys, const float * __restrict__ z, int64_t zs, const float * __restrict__ w, float eps, float mult, int n, int groups,
                                                          float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     __shared__ float red[4];
@@ -286,12 +352,12 @@ __global__ void __launch_bounds__(256) k_gate_group_norm(const float * __restric
     for (int i = threadIdx.x; i < part; i += 256) { const float g = zr[i], u = yr[i] * (g / (1.0f + expf(-g))); ss = fmaf(u, u, ss); }
     ss = pm_block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float) part + eps);
-    for (int i = threadIdx.x; i < part; i += 256) { const float g = zr[i], u = yr[i] * (g / (1.0f + expf(-g))); out[(int64_t) t * os + i0 + i] = u * inv * w[i0 + i]; }
+    for (int i = threadIdx.x; i < part; i += 256) { const float g = zr[i], u = yr[i] * (g / (1.0f + expf(-g))); out[(int64_t) t * os + i0 + i] = u * inv * w[i0 + i] * mult; }
 }
-extern "C" int pi_op_gate_group_norm(const float * y, int64_t y_stride, const float * z, int64_t z_stride, const float * w_dev, float eps, int n, int groups, int n_tok, float * out, int64_t out_stride, void * stream) {
+extern "C" int pi_op_gate_group_norm(const float * y, int64_t y_stride, const float * z, int64_t z_stride, const float * w_dev, float eps, float mult, int n, int groups, int n_tok, float * out, int64_t out_stride, void * stream) {
     if (n_tok <= 0 || n <= 0) return 0;
     if (groups < 1 || n % groups) { pi_set_error("pi_op_gate_group_norm: %d values do not divide into %d equal parts", n, groups); return -1; }
-    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 16.0 * n * n_tok, k_gate_group_norm, dim3((unsigned) n_tok, (unsigned) groups), dim3(256), 0, (hipStream_t) stream, y, y_stride, z, z_stride, w_dev, eps, n, groups, out, out_stride,
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 16.0 * n * n_tok, k_gate_group_norm, dim3((unsigned) n_tok, (unsigned) groups), dim3(256), 0, (hipStream_t) stream, y, y_stride, z, z_stride, w_dev, eps, mult, n, groups, out, out_stride,
                  pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
 }

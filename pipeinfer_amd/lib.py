@@ -164,10 +164,12 @@ def _declare(lib):
     lib.pi_rotary_table_positions.argtypes = [vp]
     lib.pi_rotary_table_free.argtypes = [vp]; lib.pi_rotary_table_free.restype = None
     lib.pi_op_qkv_prepare.argtypes = [vp, vp, vp, i64, vp, vp, f32, i32, i32, i32, i32, vp, vp, i32, vp, i64, vp, vp, vp, vp, vp]
-    lib.pi_op_chunk_attention.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, i32, f32, i32, i32, i32, i32, i32, i32, i32, vp, i64, vp, vp]
+    lib.pi_op_chunk_attention.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, i32, f32, f32, i32, i32, i32, i32, i32, i32, i32, vp, i64, vp, vp]
     lib.pi_op_causal_conv.argtypes = [vp, i64, i32, i32, vp, vp, vp, vp, i32, i32, vp, i64, vp]
     lib.pi_op_ssd_steps.argtypes = [vp, i64, vp, vp, i32, i32, vp, vp, vp]
-    lib.pi_op_gate_group_norm.argtypes = [vp, i64, vp, i64, vp, f32, i32, i32, i32, vp, i64, vp]
+    lib.pi_op_gate_group_norm.argtypes = [vp, i64, vp, i64, vp, f32, f32, i32, i32, i32, vp, i64, vp]
+    lib.pi_op_norm_chain.argtypes = [vp, i64, f32, vp, i64, f32, vp, vp, f32, i32, i32, vp, i64, vp, i64, vp, i64, i32, vp, vp, i64, vp, vp, vp, i64, vp]
+    lib.pi_op_causal_conv_steps.argtypes = [vp, i64, i32, i32, vp, vp, vp, vp, i32, i32, vp, i64, vp, i64, vp, vp, i32, vp, vp, vp]
     lib.pi_op_moe_route_groups.argtypes = [vp, vp, i64, i32, i32, i32, i32, i32, vp, vp, vp]
     lib.pi_op_moe_experts_act.argtypes = [vp, vp, i32, i32, i32, vp, i64, vp, vp, i32, i32, i32, vp, vp, i64, vp]
     lib.pi_op_moe_experts_grouped_act.argtypes = [vp, vp, i32, i32, i32, vp, i64, vp, vp, i32, i32, vp, vp, vp, vp, i64, vp]

@@ -1,7 +1,10 @@
 """Prefill and decode throughput of the Fasovik design at layer sizes of real models (random weights), beside the engine's closest GGUF model — a Llama-architecture model of the
 same width, depth and head count with Q8_0 weights, the densest quantised type the mat-vec kernels take — and the kernels' distance from the roofline for both.
 
-`bench.py --compare-hybrid [SIZE,...]` prints one JSON line per size; bench.py's default workload and line are untouched."""
+`bench.py --compare-hybrid [SIZE,...]` prints one JSON line per size; bench.py's default workload and line are untouched.
+
+`bench.py --compare-parallel [SIZE,...]` does the same for the Vikarax design (parallel mixer: chunked sigmoid attention beside a selective recurrence, gated experts with a
+shared one) beside the engine's closest model, which is Fasovik at the same width, depth, head sizes and expert sizes."""
 import ctypes as C
 import json
 import os
@@ -73,6 +76,67 @@ def write_fasovik(folder, size, seed=1):
     return folder
 
 
+# Vikarax at the sizes above: name -> key/value heads, rotated dimensions, chunk, recurrence heads x vdim, state, groups, router groups (count, keep), shared expert's ff
+VIKARAX = {
+    "w1024": (4, 32, 256, 16, 64, 64, 2, 2, 1, 512),
+    "w2048": (4, 64, 256, 32, 64, 128, 2, 2, 1, 1024),
+    "w4096": (8, 64, 512, 64, 64, 128, 4, 4, 2, 2048),
+}
+
+
+def write_random_tensors(folder, cfg, shapes, ones=(), seed=1):
+    """a model folder of random bfloat16 tensors: vectors around 0 (around 1 where the name ends in one of `ones`), matrices of unit row norm"""
+    os.makedirs(folder, exist_ok=True)
+    head, at = {}, 0
+    for name, shp in shapes.items():
+        n = int(np.prod(shp)) * 2
+        head[name] = {"dtype": "BF16", "shape": list(shp), "data_offsets": [at, at + n]}
+        at += n
+    h = json.dumps(head).encode()
+    h += b" " * (-len(h) % 8)
+    rng = np.random.default_rng(seed)
+    with open(os.path.join(folder, "model.safetensors.part"), "wb") as f:
+        f.write(struct.pack("<Q", len(h)) + h)
+        for name, shp in shapes.items():
+            if len(shp) == 1 or name.endswith(".conv"):
+                v = rng.standard_normal(shp, dtype=np.float32) * 0.1 + (1.0 if name.endswith(tuple(ones)) else 0.0)
+            else:
+                v = rng.standard_normal(shp, dtype=np.float32) * np.float32(shp[-1] ** -0.5)
+            f.write((v.view(np.uint32) >> 16).astype(np.uint16).tobytes())
+    os.replace(os.path.join(folder, "model.safetensors.part"), os.path.join(folder, "model.safetensors"))
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    return folder
+
+
+def write_vikarax(folder, size, seed=1):
+    width, n_layer, heads, dim, vdim, _, n_exp, _, top, ff, vocab = SIZES[size]
+    kv_heads, rot, chunk, r_heads, r_vdim, state, groups, g_count, g_keep, shared = VIKARAX[size]
+    inner, gn = r_heads * r_vdim, groups * state
+    layers, shapes = [], {"embed": (vocab, width), "head": (vocab, width), "final.norm": (width,), "final.norm.b": (width,)}
+    for i in range(n_layer):
+        mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": n_exp, "top": top, "groups": {"count": g_count, "keep": g_keep}}, "shared": {"ff": shared}}
+        left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "rot": {"dims": rot, "base": 10000.0}, "mask": {"size": chunk}}
+        right = {"heads": r_heads, "vdim": r_vdim, "state": state, "groups": groups, "conv": 4, "norm_groups": groups}
+        layers.append({"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 0.7, "right_scale": 0.7}, "mlp": mlp})
+        p = "l%d." % i
+        for n in ("norm1", "norm1b", "norm2", "norm2b"):
+            shapes[p + n] = shapes[p + n + ".b"] = (width,)
+        shapes[p + "dwa"] = (i + 2,)
+        q = p + "mix.left."
+        shapes.update({q + "q": (heads * dim, width), q + "k": (kv_heads * dim, width), q + "v": (kv_heads * vdim, width), q + "q.norm": (dim,), q + "k.norm": (dim,), q + "pb": (heads,),
+                       q + "g": (heads, width), q + "o": (width, heads * vdim)})
+        q = p + "mix.right."
+        shapes.update({q + "in": (2 * inner + 2 * gn + r_heads, width), q + "conv": (inner + 2 * gn, 4), q + "conv.b": (inner + 2 * gn,), q + "dt_bias": (r_heads,), q + "A_log": (r_heads,),
+                       q + "D": (r_heads,), q + "norm": (inner,), q + "o": (width, inner)})
+        shapes[p + "mlp.router"] = (n_exp, width)
+        for e in ["e%d" % e for e in range(n_exp)] + ["shared"]:
+            f = shared if e == "shared" else ff
+            shapes.update({p + "mlp.%s.gate" % e: (f, width), p + "mlp.%s.up" % e: (f, width), p + "mlp.%s.down" % e: (width, f)})
+    cfg = {"architecture": "Vikarax", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_softcap": 30.0, "layers": layers}
+    return write_random_tensors(folder, cfg, shapes, ones=("norm", "norm1", "norm2", "norm1b", "norm2b", "dwa", ".D"), seed=seed)
+
+
 class KtRow(C.Structure):          # struct pi_kt_row (include/pipeinfer_ops.h)
     _fields_ = [("family", C.c_int32), ("type", C.c_int32), ("n_tok", C.c_int32), ("sampled_dropped", C.c_int32), ("shape_bytes", C.c_uint64), ("launches", C.c_uint64),
                 ("bytes_total", C.c_double), ("sampled", C.c_uint64), ("avg_us", C.c_double), ("avg_sampled_bytes", C.c_double)]
@@ -137,6 +201,28 @@ def measure(lib, path, n_prompt, n_decode, hybrid, exact=False):
     res["decode_kernels"] = kernel_table(lib, lambda: [ctx.feed(toks[n_prompt + i:n_prompt + i + 1], n_prompt + i, 0) for i in range(8)])
     ctx.free(); model.free()
     return res
+
+
+def main_parallel(sizes, cache, n_prompt=512, n_decode=64):
+    """Vikarax beside Fasovik at equal sizes; one JSON line per size"""
+    lib = L.load()
+    L.check(lib.pi_device_init(0), "pi_device_init")
+    for size in sizes:
+        width, n_layer, heads, dim, vdim, rank, n_exp, n_id, top, ff, vocab = SIZES[size]
+        kv_heads, rot, chunk, r_heads, r_vdim, state, groups, g_count, g_keep, shared = VIKARAX[size]
+        vik, fas = os.path.join(cache, "vikarax-" + size), os.path.join(cache, "fasovik-" + size)
+        if not os.path.exists(os.path.join(vik, "model.safetensors")):
+            write_vikarax(vik, size)
+        if not os.path.exists(os.path.join(fas, "model.safetensors")):
+            write_fasovik(fas, size)
+        out = {"size": size, "config": {"width": width, "layers": n_layer, "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "rot_dims": rot, "chunk": chunk,
+                                       "recurrence": {"heads": r_heads, "vdim": r_vdim, "state": state, "groups": groups, "conv": 4}, "experts": n_exp, "top": top, "ff": ff, "shared_ff": shared,
+                                       "vocab": vocab, "n_prompt": n_prompt, "n_decode": n_decode, "fasovik": {"kv_rank": rank, "identity": n_id}},
+               "vikarax_bf16": measure(lib, vik, n_prompt, n_decode, True),
+               "fasovik_bf16": measure(lib, fas, n_prompt, n_decode, True), "data": "synthetic", "hbm_peak": HBM_PEAK}
+        print(json.dumps(out))
+        sys.stdout.flush()
+    return 0
 
 
 def main(sizes, cache, n_prompt=512, n_decode=64):

@@ -176,6 +176,34 @@ def test_layer_norm_of_one_and_of_two_inputs(n):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("n,J", [(40, 1), (320, 4), (1000, 7)])
+def test_block_end_in_one_launch(n, J):
+    """post-norm + residual into the history's last entry, the average over the history, the next pre-norm: every stage against the separate formulas, also in place"""
+    U, lib = gpu()
+    rng = np.random.default_rng(n + J)
+    T, rows = 3, 5
+    a, b, x = (rng.standard_normal((T, n)).astype(np.float32) for _ in range(3))
+    hist = rng.standard_normal((J, rows, n)).astype(np.float32)
+    w, wb, w2, w2b = (rng.standard_normal(n).astype(np.float32) for _ in range(4))
+    coef = rng.standard_normal(J).astype(np.float32)
+    ad, bd, xd, hd, cd, od = U.Dev(a), U.Dev(b), U.Dev(x), U.Dev(hist), U.Dev(coef), U.Dev(nbytes=4 * T * n)
+    ws = [U.Dev(v) for v in (w, wb, w2, w2b)]
+    y = np.stack([x[t] + O.layer_norm(a[t].astype(np.float64) + b[t], w, wb, 1e-4) for t in range(T)])
+    mixed = np.einsum("j,jtn->tn", coef[:J - 1].astype(np.float64), hist[:J - 1, :T]) + coef[J - 1] * y
+    nxt = np.stack([O.layer_norm(mixed[t], w2, w2b, 1e-4) for t in range(T)])
+    last = hd.ptr + 4 * (J - 1) * rows * n
+    L.check(lib.pi_op_norm_chain(ad.ptr, n, 1.0, bd.ptr, n, 1.0, ws[0].ptr, ws[1].ptr, 1e-4, n, T, xd.ptr, n, last, n, hd.ptr, rows * n, J, cd.ptr, xd.ptr, n, ws[2].ptr, ws[3].ptr, od.ptr, n, None))
+    h2 = hd.get(np.float32, (J, rows, n))
+    assert rel_rms(h2[J - 1, :T], y) < 2e-6 and np.array_equal(h2[:J - 1], hist[:J - 1]) and np.array_equal(h2[J - 1, T:], hist[J - 1, T:])
+    assert rel_rms(xd.get(np.float32, (T, n)), mixed) < 3e-6 and rel_rms(od.get(np.float32, (T, n)), nxt) < 5e-6
+    # without a history: the residual row is updated in place and normed for the next sublayer
+    xd = U.Dev(x)
+    L.check(lib.pi_op_norm_chain(ad.ptr, n, 0.5, None, 0, 0.0, ws[0].ptr, ws[1].ptr, 1e-4, n, T, xd.ptr, n, xd.ptr, n, None, 0, 0, None, None, 0, ws[2].ptr, ws[3].ptr, od.ptr, n, None))
+    y = np.stack([x[t] + O.layer_norm(0.5 * a[t].astype(np.float64), w, wb, 1e-4) for t in range(T)])
+    assert rel_rms(xd.get(np.float32, (T, n)), y) < 2e-6 and rel_rms(od.get(np.float32, (T, n)), np.stack([O.layer_norm(y[t], w2, w2b, 1e-4) for t in range(T)])) < 5e-6
+
+
+@pytest.mark.gpu
 def test_depth_mix_softcap_and_gated_product():
     U, lib = gpu()
     rng = np.random.default_rng(2)
@@ -257,8 +285,8 @@ def test_chunk_attention_against_explicit_sums(H, G, D, V, chunk, n_kv, T):
     dyn = np.array([0, n_kv, T, 0], np.int32)
     d = [U.Dev(a) for a in (q, kc, vc, cpos, pack_mask(vis, n_ctx), pos, pb, gate, dyn)]
     od = U.Dev(nbytes=4 * T * H * V)
-    L.check(lib.pi_op_chunk_attention(d[0].ptr, H * D + 2, d[1].ptr, d[2].ptr, d[3].ptr, d[4].ptr, d[5].ptr, d[6].ptr, d[7].ptr, H + 1, SIGMOID, 0.21, chunk, H, G, D, V, T, n_ctx, od.ptr, H * V, d[8].ptr, None))
-    got = od.get(np.float32, (T, H, V))
+    L.check(lib.pi_op_chunk_attention(d[0].ptr, H * D + 2, d[1].ptr, d[2].ptr, d[3].ptr, d[4].ptr, d[5].ptr, d[6].ptr, d[7].ptr, H + 1, SIGMOID, 0.21, -1.5, chunk, H, G, D, V, T, n_ctx, od.ptr, H * V, d[8].ptr, None))
+    got = od.get(np.float32, (T, H, V)) / np.float32(-1.5)          # (the factor on the branch's output)
     want = chunk_attention_ref(q[:, :H * D].reshape(T, H, D).astype(np.float64), np.nan_to_num(kc).astype(np.float64), np.nan_to_num(vc).astype(np.float64), cpos, vis, pos, pb.astype(np.float64),
                                gate[:, :H].astype(np.float64), 0.21, chunk, H, G)
     assert np.isfinite(got).all() and rel_rms(got, want) < 2e-5, rel_rms(got, want)
@@ -284,7 +312,7 @@ def test_chunk_border_keys_one_inside_one_outside(chunk, p):
     vis = (cpos[None, :] <= p)
     d = [U.Dev(a) for a in (q, kc, vc, cpos, pack_mask(vis, n_ctx), np.array([p], np.int32), np.full(H, -12.0, np.float32), np.array([0, n_ctx, 1, 0], np.int32))]
     od = U.Dev(nbytes=4 * H * V)
-    L.check(lib.pi_op_chunk_attention(d[0].ptr, H * D, d[1].ptr, d[2].ptr, d[3].ptr, d[4].ptr, d[5].ptr, d[6].ptr, None, 0, 0, 1.0, chunk, H, G, D, V, 1, n_ctx, od.ptr, H * V, d[7].ptr, None))
+    L.check(lib.pi_op_chunk_attention(d[0].ptr, H * D, d[1].ptr, d[2].ptr, d[3].ptr, d[4].ptr, d[5].ptr, d[6].ptr, None, 0, 0, 1.0, 1.0, chunk, H, G, D, V, 1, n_ctx, od.ptr, H * V, d[7].ptr, None))
     got = od.get(np.float32, (H, V))[0]
     assert abs(got[0] - 1.0) < 1e-3 and abs(got[1]) < 1e-3 and abs(got[2]) < 1e-3, got          # the chunk's first position counts; the one before it and the far one do not
 
@@ -303,11 +331,14 @@ def conv_ref(x, w, b, tails, rec, taps):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("taps,channels", [(4, 300), (2, 7), (3, 64), (1, 10), (7, 33)])
-def test_causal_conv_over_sequences_and_passes(taps, channels):
+@pytest.mark.parametrize("taps,channels", [(4, 300), (2, 7), (3, 64), (1, 10), (7, 33), (8, 20), (11, 9)])
+@pytest.mark.parametrize("fused", [False, True])
+def test_causal_conv_over_sequences_and_passes(taps, channels, fused):
     U, lib = gpu()
     rng = np.random.default_rng(taps * channels)
     slots = 4
+    hbv, hav = rng.standard_normal(3).astype(np.float32), rng.standard_normal(3).astype(np.float32)
+    hb, ha = U.Dev(hbv), U.Dev(hav)
     w, b = rng.standard_normal((channels, taps)).astype(np.float32), rng.standard_normal(channels).astype(np.float32)
     state = rng.standard_normal((slots, max(taps - 1, 1), channels)).astype(np.float32)          # what earlier owners left
     wd, bd, sd = U.Dev(w), U.Dev(b), U.Dev(state)
@@ -317,12 +348,20 @@ def test_causal_conv_over_sequences_and_passes(taps, channels):
         T = len(rec)
         x = rng.standard_normal((T, channels + 2)).astype(np.float32)
         xd, rd, od = U.Dev(x), U.Dev(np.array(rec, np.int32)), U.Dev(nbytes=4 * T * channels)
-        L.check(lib.pi_op_causal_conv(xd.ptr, channels + 2, channels, taps, wd.ptr, bd.ptr, sd.ptr, rd.ptr, T, SILU, od.ptr, channels, None))
+        if fused:                                                   # the entry the engine uses: one launch for short passes (with the recurrence's step sizes), the two kernels otherwise
+            raw = rng.standard_normal((T, 3)).astype(np.float32)
+            rawd, dtd, decd = U.Dev(raw), U.Dev(nbytes=4 * T * 3), U.Dev(nbytes=4 * T * 3)
+            L.check(lib.pi_op_causal_conv_steps(xd.ptr, channels + 2, channels, taps, wd.ptr, bd.ptr, sd.ptr, rd.ptr, T, SILU, od.ptr, channels, rawd.ptr, 3, hb.ptr, ha.ptr, 3, dtd.ptr, decd.ptr, None))
+            dt = O.softplus(raw.astype(np.float64) + hbv)
+            assert rel_rms(dtd.get(np.float32, (T, 3)), dt) < 1e-6 and rel_rms(decd.get(np.float32, (T, 3)), np.exp(-np.exp(hav.astype(np.float64)) * dt)) < 1e-6
+        else:
+            L.check(lib.pi_op_causal_conv(xd.ptr, channels + 2, channels, taps, wd.ptr, bd.ptr, sd.ptr, rd.ptr, T, SILU, od.ptr, channels, None))
         want = conv_ref(x[:, :channels].astype(np.float64), w.astype(np.float64), b.astype(np.float64), tails, rec, taps)
         assert rel_rms(od.get(np.float32, (T, channels)), want) < 2e-6, rec
     run([1 | F] + [1] * 9 + [3 | F] + [0 | F, 0])                   # three sequences start: ten tokens, one token, two tokens
     run([3] + [0] + [1, 1])                                        # ... and go on with fewer tokens than taps: old and new inputs mix in the window
     run([3, 3] + [0] * 12)
+    run([0] * 20 + [3] * 25)                                        # more than 32 tokens: the fused entry takes the two-kernel path
     run([1])
     run([1 | F] + [1] * 3 + [3])                                   # slot 1 handed to a new sequence
     if taps > 1:
@@ -402,9 +441,9 @@ def test_gate_then_norm_in_parts(n, groups):
     T = 3
     y, z, w = rng.standard_normal((T, n + 1)).astype(np.float32), rng.standard_normal((T, n + 5)).astype(np.float32), rng.standard_normal(n).astype(np.float32)
     yd, zd, wd = U.Dev(y), U.Dev(z), U.Dev(w)
-    L.check(lib.pi_op_gate_group_norm(yd.ptr, n + 1, zd.ptr, n + 5, wd.ptr, 1e-3, n, groups, T, yd.ptr, n + 1, None))          # in place, as the engine calls it
+    L.check(lib.pi_op_gate_group_norm(yd.ptr, n + 1, zd.ptr, n + 5, wd.ptr, 1e-3, 0.6, n, groups, T, yd.ptr, n + 1, None))     # in place, as the engine calls it
     u = y[:, :n].astype(np.float64) * O.silu(z[:, :n].astype(np.float64))
-    want = np.stack([np.concatenate([O.unit_rms(part, 1e-3) for part in u[t].reshape(groups, -1)]) * w for t in range(T)])
+    want = np.stack([np.concatenate([O.unit_rms(part, 1e-3) for part in u[t].reshape(groups, -1)]) * w * 0.6 for t in range(T)])
     got = yd.get(np.float32, (T, n + 1))
     assert rel_rms(got[:, :n], want) < 2e-6 and np.array_equal(got[:, n], y[:, n])
 

@@ -5,8 +5,8 @@
 //   k_linear_attention   per head S <- lambda * S + k v^T, o = S^T q over a run of tokens of one sequence; S lives in HBM per (slot, head) between calls
 //   k_latent_attention   attention over a shared low-rank latent c: the key up-projection is folded into the query (q~ = W_uk^T q), the value up-projection applied to the
 //                        probability-weighted sum of latents — the cache is read once for all heads of a tile and K / V are never materialised; soft-max with a sink term
-//   k_layer_norm_mix     y = ((ca * a + cb * b) - mean) / sqrt(variance + eps) * w + bias;  out = [residual +] y   (the norm behind a sublayer with two branches)
-//   k_norm_chain         the three row operations at the end of a block in one launch: post-norm + residual, the depth average, the next sublayer's pre-norm
+//   k_norm_chain(_reg)   y = ((ca * a + cb * b) - mean) / sqrt(variance + eps) * w + bias;  out = [residual +] y   (layer norm of one input or of the weighted sum of two), and
+//                        the three row operations at the end of a block in one launch: post-norm + residual, the depth average, the next sublayer's pre-norm
 //   k_depth_mix          out = sum_j coef[j] * X_j over the stream's earlier states (a learned average over depth)
 //   k_moe_route          router logits, soft-max over all router outputs, bias-corrected top-k choice, weights = uncorrected scores
 //   k_moe_up / _down     the chosen experts of every token (gathered mat-vecs), identity experts pass their input through
@@ -104,36 +104,7 @@ extern "C" int pi_op_rms_scale(const float * x, int64_t x_stride, const float * 
     PI_CHECK_LAUNCH(); return 0;
 }
 
-// ---- layer norm (weight and bias) over one or the weighted sum of two inputs, optional residual ---------------------------------------------------------------
-// two passes over the row for the statistics (mean, then the mean of squared deviations), a third for the output: the row stays in L2 / registers' reach
-__global__ void __launch_bounds__(256) k_layer_norm_mix(const float * __restrict__ a, int64_t as, float ca, const float * __restrict__ b, int64_t bs, float cb, const float * __restrict__ w,
-                                                        const float * __restrict__ bias, float eps, int n, const float * __restrict__ res, int64_t rs, float * __restrict__ out, int64_t os,
-                                                        const int32_t * __restrict__ abort_w) {
-    if (pi_aborted(abort_w)) return;
-    __shared__ float red[4];
-    const int t = blockIdx.x;
-    const float * ar = a + (int64_t) t * as, * br = b ? b + (int64_t) t * bs : nullptr;
-    auto val = [&](int i) { const float v = ca * ar[i]; return br ? fmaf(cb, br[i], v) : v; };
-    float sum = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) sum += val(i);
-    const float mean = hy_block_sum(sum, red) / (float) n;
-    float ss = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) { const float d = val(i) - mean; ss = fmaf(d, d, ss); }
-    const float inv = 1.0f / sqrtf(hy_block_sum(ss, red) / (float) n + eps);
-    for (int i = threadIdx.x; i < n; i += 256) {
-        float y = (val(i) - mean) * inv * w[i] + (bias ? bias[i] : 0.0f);
-        if (res) y = res[(int64_t) t * rs + i] + y;
-        out[(int64_t) t * os + i] = y;
-    }
-}
-extern "C" int pi_op_layer_norm_mix(const float * a, int64_t a_stride, float ca, const float * b, int64_t b_stride, float cb, const float * w_dev, const float * bias_dev, float eps, int n, int n_tok,
-                                    const float * residual, int64_t residual_stride, float * out, int64_t out_stride, void * stream) {
-    if (n_tok <= 0 || n <= 0) return 0;
-    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 4.0 * n * n_tok * (2.0 + (b ? 1 : 0) + (residual ? 1 : 0)), k_layer_norm_mix, dim3((unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, a, a_stride, ca, b, b_stride, cb,
-                 w_dev, bias_dev, eps, n, residual, residual_stride, out, out_stride, pi_abort_word());
-    PI_CHECK_LAUNCH(); return 0;
-}
-
+// ---- layer norm (weight and bias) over one or the weighted sum of two inputs, optional residual; the row operations at the end of a block -----------------------------
 // The end of a block as one launch, per token row:  v = [residual +] LN_A(ca * a + cb * b)  -> out_a;   (n_hist > 0)  v = sum_(j < n_hist - 1) coef[j] * hist[j] + coef[n_hist - 1] * v
 // -> out_mix  (out_a is hist[n_hist - 1]: the block's result joins the history it is averaged with);   (w_c)  LN_C(v) -> out_c  (the next sublayer's input).
 // A thread re-reads only what it wrote itself, so no barrier is needed between the stages beyond those of the sums.
@@ -175,6 +146,63 @@ __global__ void __launch_bounds__(256) k_norm_chain(const float * __restrict__ a
     const float inv_c = 1.0f / sqrtf(hy_block_sum(ss_c, red) / (float) n + eps);
     for (int i = threadIdx.x; i < n; i += 256) out_c[(int64_t) t * ocs + i] = (last[i] - mean_c) * inv_c * w_c[i] + (bias_c ? bias_c[i] : 0.0f);
 }
+// The same with the row in registers (n <= 256 * NPT): every input is loaded once, all loads are issued before the first sum, and the stages only exchange their sums
+template <int NPT>
+__global__ void __launch_bounds__(256) k_norm_chain_reg(const float * __restrict__ a, int64_t as, float ca, const float * __restrict__ b, int64_t bs, float cb, const float * __restrict__ w,
+                                                        const float * __restrict__ bias, float eps, int n, const float * __restrict__ res, int64_t rs, float * __restrict__ out_a, int64_t oas,
+                                                        const float * __restrict__ hist, int64_t hist_stride, int n_hist, const float * __restrict__ coef, float * __restrict__ out_mix, int64_t oms,
+                                                        const float * __restrict__ w_c, const float * __restrict__ bias_c, float * __restrict__ out_c, int64_t ocs, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    __shared__ float red[4];
+    const int t = blockIdx.x;
+    const float * ar = a + (int64_t) t * as, * br = b ? b + (int64_t) t * bs : nullptr;
+    float v[NPT], wv[NPT], bv[NPT], rv[NPT], mv[NPT];
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NPT; k++) {
+        const int i = threadIdx.x + k * 256;
+        const bool ok = i < n;
+        float x = ok ? ca * ar[i] : 0.0f;
+        if (ok && br) x = fmaf(cb, br[i], x);
+        v[k] = x; sum += x;
+        wv[k] = ok ? w[i] : 0.0f; bv[k] = ok && bias ? bias[i] : 0.0f; rv[k] = ok && res ? res[(int64_t) t * rs + i] : 0.0f;
+        float m = 0.0f;
+        if (ok) for (int j = 0; j < n_hist - 1; j++) m = fmaf(coef[j], hist[(int64_t) j * hist_stride + (int64_t) t * n + i], m);
+        mv[k] = m;
+    }
+    const float mean = hy_block_sum(sum, red) / (float) n;
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NPT; k++) if (threadIdx.x + k * 256 < n) { const float d = v[k] - mean; ss = fmaf(d, d, ss); }
+    const float inv = 1.0f / sqrtf(hy_block_sum(ss, red) / (float) n + eps);
+    const float c_last = n_hist > 0 ? coef[n_hist - 1] : 0.0f;
+    float sum_c = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NPT; k++) {
+        const int i = threadIdx.x + k * 256;
+        if (i < n) {
+            float y = (v[k] - mean) * inv * wv[k] + bv[k];
+            if (res) y = rv[k] + y;
+            out_a[(int64_t) t * oas + i] = y;
+            if (n_hist > 0) { y = fmaf(c_last, y, mv[k]); out_mix[(int64_t) t * oms + i] = y; }
+            v[k] = y; sum_c += y;
+        }
+    }
+    if (!w_c) return;
+#pragma unroll
+    for (int k = 0; k < NPT; k++) { const int i = threadIdx.x + k * 256; wv[k] = i < n ? w_c[i] : 0.0f; bv[k] = i < n && bias_c ? bias_c[i] : 0.0f; }
+    const float mean_c = hy_block_sum(sum_c, red) / (float) n;
+    float ss_c = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NPT; k++) if (threadIdx.x + k * 256 < n) { const float d = v[k] - mean_c; ss_c = fmaf(d, d, ss_c); }
+    const float inv_c = 1.0f / sqrtf(hy_block_sum(ss_c, red) / (float) n + eps);
+#pragma unroll
+    for (int k = 0; k < NPT; k++) { const int i = threadIdx.x + k * 256; if (i < n) out_c[(int64_t) t * ocs + i] = (v[k] - mean_c) * inv_c * wv[k] + bv[k]; }
+}
+extern "C" int pi_op_layer_norm_mix(const float * a, int64_t a_stride, float ca, const float * b, int64_t b_stride, float cb, const float * w_dev, const float * bias_dev, float eps, int n, int n_tok,
+                                    const float * residual, int64_t residual_stride, float * out, int64_t out_stride, void * stream) {
+    return pi_op_norm_chain(a, a_stride, ca, b, b_stride, cb, w_dev, bias_dev, eps, n, n_tok, residual, residual_stride, out, out_stride, nullptr, 0, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, 0, stream);
+}
 extern "C" int pi_op_norm_chain(const float * a, int64_t a_stride, float ca, const float * b, int64_t b_stride, float cb, const float * w_dev, const float * bias_dev, float eps, int n, int n_tok,
                                 const float * residual, int64_t residual_stride, float * out_a, int64_t out_a_stride, const float * hist, int64_t hist_stride, int n_hist, const float * coef_dev,
                                 float * out_mix, int64_t out_mix_stride, const float * w_next, const float * bias_next, float * out_next, int64_t out_next_stride, void * stream) {
@@ -183,8 +211,11 @@ extern "C" int pi_op_norm_chain(const float * a, int64_t a_stride, float ca, con
         pi_set_error("pi_op_norm_chain: the block's result must be written into the last entry of the history it is averaged with"); return -1;
     }
     if (w_next && (!out_next || out_next == out_a || out_next == out_mix)) { pi_set_error("pi_op_norm_chain: the next norm needs an output of its own"); return -1; }
-    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 4.0 * n * n_tok * (3.0 + (b ? 1 : 0) + (residual ? 1 : 0) + n_hist + (w_next ? 2 : 0)), k_norm_chain, dim3((unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, a, a_stride, ca, b, b_stride, cb,
-                 w_dev, bias_dev, eps, n, residual, residual_stride, out_a, out_a_stride, hist, hist_stride, n_hist, coef_dev, out_mix, out_mix_stride, w_next, bias_next, out_next, out_next_stride, pi_abort_word());
+    const double bytes = 4.0 * n * n_tok * (3.0 + (b ? 1 : 0) + (residual ? 1 : 0) + n_hist + (w_next ? 2 : 0));
+#define NC_GO(K) PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, bytes, K, dim3((unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, a, a_stride, ca, b, b_stride, cb, w_dev, bias_dev, eps, n, residual, residual_stride, \
+                              out_a, out_a_stride, hist, hist_stride, n_hist, coef_dev, out_mix, out_mix_stride, w_next, bias_next, out_next, out_next_stride, pi_abort_word())
+    if (n <= 1024) NC_GO(k_norm_chain_reg<4>); else if (n <= 2048) NC_GO(k_norm_chain_reg<8>); else if (n <= 4096) NC_GO(k_norm_chain_reg<16>); else if (n <= 8192) NC_GO(k_norm_chain_reg<32>); else NC_GO(k_norm_chain);
+#undef NC_GO
     PI_CHECK_LAUNCH(); return 0;
 }
 

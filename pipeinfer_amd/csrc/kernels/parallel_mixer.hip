@@ -107,6 +107,24 @@ extern "C" int pi_op_qkv_prepare(const float * q, const float * k, const float *
 // grid (token, key / value head): the workgroup serves the `hpg` query heads of its key head.  The cells are walked 256 at a time; the visible ones of a block are compacted
 // in cell order (so that the sum has one order whatever the launch), their key rows staged in LDS 64 at a time.  Scores: thread (cell, query head); output: thread (query
 // head, value column), value rows read from the cache along the columns.
+// rows `cells[0 .. nl)` of a cache [cells][G][W] (head g) into LDS rows `pitch` floats apart.  Sixteen loads per thread are issued before the first LDS store: the compiler cannot
+// tell the cell list (LDS) from the tile (LDS) and would otherwise wait for every row's trip to memory before it reads the next cell number
+static __device__ __forceinline__ void ca_stage(const float * __restrict__ cache, const int * cells, int nl, int G, int g, int W, int pitch, float * tile, int tid) {
+    const int total = nl * W;
+    for (int base = 0; base < total; base += 256 * 16) {
+        float tmp[16];
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            const int i = base + u * 256 + tid;
+            tmp[u] = i < total ? cache[((int64_t) cells[i / W] * G + g) * W + i % W] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            const int i = base + u * 256 + tid;
+            if (i < total) tile[(i / W) * pitch + i % W] = tmp[u];
+        }
+    }
+}
 #define CA_TILE 64                                // key rows staged at a time (fewer when a row is long: ca_tile)
 #define CA_MAXOUT 16                              // outputs (query head, value column) a thread accumulates: hpg * vdim <= 256 * CA_MAXOUT
 __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * __restrict__ kc, const float * __restrict__ vc, const int32_t * __restrict__ cell_pos,
@@ -114,11 +132,11 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
                                                          float scale, float out_mult, int chunk, int H, int G, int D, int V, int n_kv_arg, int tile, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
                                                          const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
-    extern __shared__ float lds[];                // q [hpg][D] | key tile [tile][D + 1] | weights [tile][hpg]
+    extern __shared__ float lds[];                // q [hpg][D] | key tile [tile][D + 1], then the value tile [tile][V] in the same place | weights [tile][hpg]
     __shared__ int list[256], wcnt[4];
     const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hpg = H / G, h0 = g * hpg, DP = D + 1;
-    float * qsh = lds, * ksh = qsh + hpg * D, * wsh = ksh + tile * DP;
+    float * qsh = lds, * ksh = qsh + hpg * D, * wsh = ksh + tile * max(DP, V);
     const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg);
     const int words = (n_kv_arg + 31) / 32;
     const uint32_t * mrow = mask + (int64_t) t * words;
@@ -145,8 +163,8 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
         __syncthreads();
         for (int l0 = 0; l0 < total; l0 += tile) {
             const int nl = min(tile, total - l0);
-            if (l0) __syncthreads();
-            for (int i = tid; i < nl * D; i += 256) { const int cc = i / D, d = i % D; ksh[cc * DP + d] = kc[((int64_t) list[l0 + cc] * G + g) * D + d]; }
+            if (l0) __syncthreads();                 // (the previous tile's values are no longer read)
+            ca_stage(kc, list + l0, nl, G, g, D, DP, ksh, tid);
             __syncthreads();
             for (int i = tid; i < nl * hpg; i += 256) {
                 const int cc = i % nl, m = i / nl;
@@ -156,13 +174,16 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
                 wsh[cc * hpg + m] = pm_sigmoid(s * scale + (hbias ? hbias[h0 + m] : 0.0f));
             }
             __syncthreads();
+            // the value rows take the key tile's place: all their loads are in flight together (read one by one in the sum below, every row would cost a trip to memory)
+            ca_stage(vc, list + l0, nl, G, g, V, V, ksh, tid);
+            __syncthreads();
 #pragma unroll
             for (int oi = 0; oi < CA_MAXOUT; oi++) {
                 const int o = oi * 256 + tid;
                 if (o < n_out) {
                     const int m = o / V, vv = o % V;
                     float a = acc[oi];
-                    for (int cc = 0; cc < nl; cc++) a = fmaf(wsh[cc * hpg + m], vc[((int64_t) list[l0 + cc] * G + g) * V + vv], a);
+                    for (int cc = 0; cc < nl; cc++) a = fmaf(wsh[cc * hpg + m], ksh[cc * V + vv], a);
                     acc[oi] = a;
                 }
             }
@@ -187,7 +208,7 @@ extern "C" int pi_op_chunk_attention(const float * q, int64_t q_stride, const fl
     if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || vdim < 1 || chunk < 0) { pi_set_error("pi_op_chunk_attention: %d query heads over %d key / value heads, sizes %d / %d, chunk %d", heads, kv_heads, dim, vdim, chunk); return -1; }
     const int hpg = heads / kv_heads;
     int tile = CA_TILE;
-    auto lds_of = [&](int tl) { return ((size_t) hpg * dim + (size_t) tl * (dim + 1) + (size_t) tl * hpg) * sizeof(float); };
+    auto lds_of = [&](int tl) { return ((size_t) hpg * dim + (size_t) tl * std::max(dim + 1, vdim) + (size_t) tl * hpg) * sizeof(float); };
     while (tile > 4 && lds_of(tile) > 60 * 1024) tile >>= 1;
     const size_t lds = lds_of(tile);
     if (hpg * vdim > 256 * CA_MAXOUT || lds > 60 * 1024) { pi_set_error("pi_op_chunk_attention: %d query heads per key head of sizes %d / %d are beyond the kernel (LDS %zu bytes)", hpg, dim, vdim, lds); return -1; }

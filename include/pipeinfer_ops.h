@@ -192,6 +192,7 @@ PI_API int pi_op_linear_attention(const float * q_dev, const float * k_dev, cons
                                   const int32_t * rec_dev, int n_tok, int max_segments, float * scratch_dev, size_t scratch_floats, float * out_dev, int64_t out_stride, void * stream);
 /* passes of more than 32 tokens cut the sequences into pieces that run side by side (the recurrence is linear in the state): floats of scratch they need (0 for shorter passes) */
 PI_API size_t pi_op_linear_attention_scratch_floats(int heads, int dim, int vdim, int n_tok, int max_segments);
+PI_API int pi_op_linear_attention_reserve(void);                   /* once per process, outside graph capture: the LDS limit wide keys need */
 PI_API int pi_op_copy_f32(const float * src_dev, float * dst_dev, int64_t n, void * stream);
 /* Attention over a cache of latents c [cells][rank] fp32 shared by all heads: k = W_uk c, v = W_uv c per head, never materialised (W_uk is folded into the query, W_uv applied to
  * the weighted sum of latents); score = q . k * scale; soft-max whose denominator also holds exp(sink[h]).  mask_dev / n_kv / dyn_dev as for pi_op_attention_ex (single run).

@@ -144,7 +144,7 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
         if (hipStreamCreateWithFlags(&ctx->ctl_stream, hipStreamNonBlocking) != hipSuccess) { err = "hipStreamCreate(control) failed"; return false; }
     }
     ctx->use_graphs = ctx->use_graphs && getenv("PI_NO_GRAPHS") == nullptr;
-    if (pi_op_latent_attention_reserve() != 0) { err = pi_last_error(); return false; }
+    if (pi_op_latent_attention_reserve() != 0 || (hp.n_recurrent() > 0 && pi_op_linear_attention_reserve() != 0)) { err = pi_last_error(); return false; }
     ctx->mask_cap_words = (size_t) nb * ((ctx->n_ctx + 31) / 32);
     if (!(ctx->mask_dev = (uint32_t *) dev(ctx->mask_cap_words * 4))) return false;
     if (!(ctx->logits_dev = (float *) dev((size_t) 4 * nb * hp.n_vocab)) || !(ctx->topk_ids_dev = (int32_t *) dev((size_t) 4 * nb * 8)) ||

@@ -442,6 +442,17 @@ __global__ void __launch_bounds__(256) k_linear_state_scan(int heads, int dim, i
     }
 }
 
+// once per process, outside graph capture: the tiles of wide keys (q, k of 32 tokens) need more dynamic LDS than a kernel gets by default
+#define LA_LDS_MAX (150 * 1024)
+extern "C" int pi_op_linear_attention_reserve(void) {
+    static bool done = false;
+    if (done) return 0;
+    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_linear_attention<8>, hipFuncAttributeMaxDynamicSharedMemorySize, LA_LDS_MAX));
+    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_linear_attention<16>, hipFuncAttributeMaxDynamicSharedMemorySize, LA_LDS_MAX));
+    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_linear_attention<32>, hipFuncAttributeMaxDynamicSharedMemorySize, LA_LDS_MAX));
+    done = true;
+    return 0;
+}
 static int la_max_pieces(int n_tok, int max_segments) { return n_tok / LA_TB + std::min(n_tok, std::max(1, max_segments)) + 1; }
 extern "C" size_t pi_op_linear_attention_scratch_floats(int heads, int dim, int vdim, int n_tok, int max_segments) {
     return n_tok <= LA_TB ? 0 : (size_t) la_max_pieces(n_tok, max_segments) * heads * dim * vdim;
@@ -468,6 +479,8 @@ extern "C" int pi_op_linear_attention_ex(const float * q, const float * k, const
     const unsigned gz = pieces ? (unsigned) la_max_pieces(n_tok, max_segments) : (unsigned) std::max(1, std::min(n_tok, max_segments));
     const dim3 grid((unsigned) heads, (unsigned) ((vdim + cols - 1) / cols), gz);
     const size_t lds = ((size_t) 2 * LA_TB * dim + (size_t) LA_TB * cols + (size_t) n_tok) * sizeof(float);
+    if (lds > LA_LDS_MAX) { pi_set_error("pi_op_linear_attention: a key width of %d with %d tokens in the pass needs %zu bytes of LDS (at most %d)", dim, n_tok, lds, LA_LDS_MAX); return -1; }
+    if (lds > 48 * 1024 && pi_op_linear_attention_reserve() != 0) return -1;
     const double bytes = 4.0 * n_tok * heads * (2.0 * dim + 2.0 * vdim) + 8.0 * heads * dim * vdim;
     hipStream_t s = (hipStream_t) stream;
     const int nta = std::min(n_tok, PI_KT_MAXNT - 1);

@@ -382,7 +382,7 @@ def ssd_ref(C_, B, x, dt, decay, D, S, heads, groups):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("heads,groups,N,P", [(4, 2, 6, 5), (1, 1, 48, 48), (6, 3, 16, 70), (8, 1, 100, 12), (2, 2, 130, 33)])
+@pytest.mark.parametrize("heads,groups,N,P", [(4, 2, 6, 5), (1, 1, 48, 48), (6, 3, 16, 70), (8, 1, 100, 12), (2, 2, 130, 33), (1, 1, 300, 8)])
 def test_selective_recurrence_steps_groups_and_long_passes(heads, groups, N, P):
     """dt and the decays from raw values; then the recurrence with per-token decays, keys scaled by dt, B / C shared inside a group, the skip term; passes longer than the
     32-token pieces (states chained across pieces), several sequences per pass, carried and fresh states"""

@@ -104,28 +104,49 @@ extern "C" int pi_op_qkv_prepare(const float * q, const float * k, const float *
 }
 
 // ---- attention with sigmoid weights inside chunks ---------------------------------------------------------------------------------------------------------
-// grid (token, key / value head): the workgroup serves the `hpg` query heads of its key head.  The cells are walked 256 at a time; the visible ones of a block are compacted
+// grid (token, key / value head): the workgroup serves the `hpg` query heads of its key head.  The cells are walked 256 at a time; the visible ones of a round are compacted
 // in cell order (so that the sum has one order whatever the launch), their key rows staged in LDS 64 at a time.  Scores: thread (cell, query head); output: thread (query
 // head, value column), value rows read from the cache along the columns.
-// rows `cells[0 .. nl)` of a cache [cells][G][W] (head g) into LDS rows `pitch` floats apart.  Sixteen loads per thread are issued before the first LDS store: the compiler cannot
+// rows `cells[0 .. nl)` of a cache [cells][G][W] (head g) into LDS rows `pitch` floats apart.  Eight loads per thread are issued before the first LDS store: the compiler cannot
 // tell the cell list (LDS) from the tile (LDS) and would otherwise wait for every row's trip to memory before it reads the next cell number
 static __device__ __forceinline__ void ca_stage(const float * __restrict__ cache, const int * cells, int nl, int G, int g, int W, int pitch, float * tile, int tid) {
-    const int total = nl * W;
-    for (int base = 0; base < total; base += 256 * 16) {
-        float tmp[16];
+    const int lane = tid & 63, wave = tid >> 6;
+    if (W <= 128) {                                                   // a wave per row, two columns per lane, four rows per round: no index arithmetic beyond adds
+        for (int r0 = wave; r0 < nl; r0 += 16) {
+            float tmp[8];
 #pragma unroll
-        for (int u = 0; u < 16; u++) {
+            for (int u = 0; u < 4; u++) {
+                const int cc = r0 + u * 4;
+                const float * row = cache + ((int64_t) cells[min(cc, nl - 1)] * G + g) * W;
+                tmp[2 * u] = cc < nl && lane < W ? row[lane] : 0.0f;
+                tmp[2 * u + 1] = cc < nl && lane + 64 < W ? row[lane + 64] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int cc = r0 + u * 4;
+                if (cc < nl && lane < W) tile[cc * pitch + lane] = tmp[2 * u];
+                if (cc < nl && lane + 64 < W) tile[cc * pitch + lane + 64] = tmp[2 * u + 1];
+            }
+        }
+        return;
+    }
+    const int total = nl * W;
+    for (int base = 0; base < total; base += 256 * 8) {
+        float tmp[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
             const int i = base + u * 256 + tid;
             tmp[u] = i < total ? cache[((int64_t) cells[i / W] * G + g) * W + i % W] : 0.0f;
         }
 #pragma unroll
-        for (int u = 0; u < 16; u++) {
+        for (int u = 0; u < 8; u++) {
             const int i = base + u * 256 + tid;
             if (i < total) tile[(i / W) * pitch + i % W] = tmp[u];
         }
     }
 }
 #define CA_TILE 64                                // key rows staged at a time (fewer when a row is long: ca_tile)
+#define CA_SB 1                                   // blocks of 256 cells whose visibility is worked out in one round
 #define CA_MAXOUT 16                              // outputs (query head, value column) a thread accumulates: hpg * vdim <= 256 * CA_MAXOUT
 __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * __restrict__ kc, const float * __restrict__ vc, const int32_t * __restrict__ cell_pos,
                                                          const uint32_t * __restrict__ mask, const int32_t * __restrict__ pos, const float * __restrict__ hbias, const float * __restrict__ gate, int64_t gs, int gate_act,
@@ -133,7 +154,7 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
                                                          const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
     extern __shared__ float lds[];                // q [hpg][D] | key tile [tile][D + 1], then the value tile [tile][V] in the same place | weights [tile][hpg]
-    __shared__ int list[256], wcnt[4];
+    __shared__ int list[256 * CA_SB], wcnt[4 * CA_SB];
     const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hpg = H / G, h0 = g * hpg, DP = D + 1;
     float * qsh = lds, * ksh = qsh + hpg * D, * wsh = ksh + tile * max(DP, V);
@@ -147,19 +168,31 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
 #pragma unroll
     for (int i = 0; i < CA_MAXOUT; i++) acc[i] = 0.0f;
     const int n_out = hpg * V;
-    for (int c0 = 0; c0 < n_kv; c0 += 256) {
-        const int c = c0 + tid;
-        bool vis = false;
-        if (c < n_kv && ((mrow[c >> 5] >> (c & 31)) & 1u)) vis = cell_pos[c] >= first_pos;
-        const unsigned long long b = __ballot(vis);
-        __syncthreads();                          // (the previous block's list and tiles are no longer read)
-        if (lane == 0) wcnt[wave] = __popcll(b);
+    for (int c0 = 0; c0 < n_kv; c0 += 256 * CA_SB) {                 // CA_SB blocks of 256 cells at a time: their mask words and positions are loaded together
+        bool vis[CA_SB]; unsigned long long bal[CA_SB];
+#pragma unroll
+        for (int u = 0; u < CA_SB; u++) {
+            const int c = c0 + u * 256 + tid;
+            const bool in = c < n_kv;
+            const uint32_t word = in ? mrow[c >> 5] : 0u;
+            const int cp = in ? cell_pos[c] : -1;
+            vis[u] = in && ((word >> (c & 31)) & 1u) && cp >= first_pos;
+        }
+#pragma unroll
+        for (int u = 0; u < CA_SB; u++) bal[u] = __ballot(vis[u]);
+        __syncthreads();                          // (the previous round's list and tiles are no longer read)
+        if (lane == 0)
+#pragma unroll
+            for (int u = 0; u < CA_SB; u++) wcnt[u * 4 + wave] = __popcll(bal[u]);
         __syncthreads();
-        const int total = wcnt[0] + wcnt[1] + wcnt[2] + wcnt[3];
+        int total = 0, mine[CA_SB];               // cell order: block, then wave, then lane
+#pragma unroll
+        for (int u = 0; u < CA_SB; u++)
+#pragma unroll
+            for (int w = 0; w < 4; w++) { if (w == wave) mine[u] = total; total += wcnt[u * 4 + w]; }
         if (total == 0) continue;
-        int at = 0;
-        for (int w = 0; w < wave; w++) at += wcnt[w];
-        if (vis) list[at + __popcll(b & ((1ull << lane) - 1ull))] = c;
+#pragma unroll
+        for (int u = 0; u < CA_SB; u++) if (vis[u]) list[mine[u] + __popcll(bal[u] & ((1ull << lane) - 1ull))] = c0 + u * 256 + tid;
         __syncthreads();
         for (int l0 = 0; l0 < total; l0 += tile) {
             const int nl = min(tile, total - l0);

@@ -245,3 +245,38 @@ def main(sizes, cache, n_prompt=512, n_decode=64):
         print(json.dumps(out))
         sys.stdout.flush()
     return 0
+
+
+def run_phase(design, size, phase, cache, n_prompt=512, n_decode=64):
+    """one phase of one design at one size and nothing else, for a profiler: `prefill` = four prompt passes, `decode` = one prompt pass and n_decode single tokens"""
+    lib = L.load()
+    L.check(lib.pi_device_init(0), "pi_device_init")
+    folder = os.path.join(cache, "%s-%s" % (design, size))
+    if not os.path.exists(os.path.join(folder, "model.safetensors")):
+        (write_vikarax if design == "vikarax" else write_fasovik)(folder, size)
+    model = LL.Model(folder)
+    ctx = LL.Context(model, n_ctx=n_prompt + n_decode + 64, n_batch=n_prompt)
+    ctx.set_precision(False)
+    rng = np.random.default_rng(7)
+    toks = [int(t) for t in rng.integers(1, model.n_vocab, n_prompt + n_decode)]
+    if phase == "prefill":
+        for _ in range(4):
+            ctx.feed(toks[:n_prompt], 0, 0)
+            ctx.seq_rm(0, -1, -1)
+    else:
+        ctx.feed(toks[:n_prompt], 0, 0)
+        for i in range(n_decode):
+            ctx.feed(toks[n_prompt + i:n_prompt + i + 1], n_prompt + i, 0)
+    ctx.free(); model.free()
+    return 0
+
+
+if __name__ == "__main__":
+    import argparse
+    ap = argparse.ArgumentParser(description="one phase of one folder-described design at one size (for `rocprofv3 --kernel-trace --stats -- python3 -m pipeinfer_amd.tools.hybrid_bench ...`)")
+    ap.add_argument("--design", choices=["vikarax", "fasovik"], required=True)
+    ap.add_argument("--size", choices=sorted(SIZES), default="w2048")
+    ap.add_argument("--phase", choices=["prefill", "decode"], required=True)
+    ap.add_argument("--cache", default=os.environ.get("PIPEINFER_CACHE", "/tmp/pipeinfer_models"))
+    a = ap.parse_args()
+    sys.exit(run_phase(a.design, a.size, a.phase, a.cache))

@@ -104,7 +104,7 @@ extern "C" int pi_op_qkv_prepare(const float * q, const float * k, const float *
 }
 
 // ---- attention with sigmoid weights inside chunks ---------------------------------------------------------------------------------------------------------
-// grid (token, key / value head): the workgroup serves the `hpg` query heads of its key head.  The cells are walked 256 at a time; the visible ones of a round are compacted
+// grid (token, key / value head, split of its query heads): the workgroup serves the query heads of its key head (all of them in one workgroup unless they are very many or very wide).  The cells are walked 256 at a time; the visible ones of a round are compacted
 // in cell order (so that the sum has one order whatever the launch), their key rows staged in LDS 64 at a time.  Scores: thread (cell, query head); output: thread (query
 // head, value column), value rows read from the cache along the columns.
 // rows `cells[0 .. nl)` of a cache [cells][G][W] (head g) into LDS rows `pitch` floats apart.  Eight loads per thread are issued before the first LDS store: the compiler cannot
@@ -150,13 +150,13 @@ static __device__ __forceinline__ void ca_stage(const float * __restrict__ cache
 #define CA_MAXOUT 16                              // outputs (query head, value column) a thread accumulates: hpg * vdim <= 256 * CA_MAXOUT
 __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * __restrict__ kc, const float * __restrict__ vc, const int32_t * __restrict__ cell_pos,
                                                          const uint32_t * __restrict__ mask, const int32_t * __restrict__ pos, const float * __restrict__ hbias, const float * __restrict__ gate, int64_t gs, int gate_act,
-                                                         float scale, float out_mult, int chunk, int H, int G, int D, int V, int n_kv_arg, int tile, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
+                                                         float scale, float out_mult, int chunk, int H, int G, int D, int V, int n_kv_arg, int tile, int hps, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
                                                          const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
     extern __shared__ float lds[];                // q [hpg][D] | key tile [tile][D + 1], then the value tile [tile][V] in the same place | weights [tile][hpg]
     __shared__ int list[256 * CA_SB], wcnt[4 * CA_SB];
     const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int hpg = H / G, h0 = g * hpg, DP = D + 1;
+    const int hs = blockIdx.z * hps, hpg = min(hps, H / G - hs), h0 = g * (H / G) + hs, DP = D + 1;        // this workgroup's query heads: hpg of them from h0 on (all of the key head's unless they are split over blockIdx.z)
     float * qsh = lds, * ksh = qsh + hpg * D, * wsh = ksh + tile * max(DP, V);
     const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg);
     const int words = (n_kv_arg + 31) / 32;
@@ -239,7 +239,8 @@ extern "C" int pi_op_chunk_attention(const float * q, int64_t q_stride, const fl
                                      float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
     if (n_tok <= 0) return 0;
     if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || vdim < 1 || chunk < 0) { pi_set_error("pi_op_chunk_attention: %d query heads over %d key / value heads, sizes %d / %d, chunk %d", heads, kv_heads, dim, vdim, chunk); return -1; }
-    const int hpg = heads / kv_heads;
+    int hpg = heads / kv_heads, splits = 1;                            // query heads of a key head that one workgroup serves: all of them, unless their outputs or the LDS plan say otherwise
+    while (hpg > 1 && (hpg * vdim > 256 * CA_MAXOUT || (size_t) hpg * dim * sizeof(float) > 24 * 1024)) { splits *= 2; hpg = (heads / kv_heads + splits - 1) / splits; }
     int tile = CA_TILE;
     auto lds_of = [&](int tl) { return ((size_t) hpg * dim + (size_t) tl * std::max(dim + 1, vdim) + (size_t) tl * hpg) * sizeof(float); };
     while (tile > 4 && lds_of(tile) > 60 * 1024) tile >>= 1;
@@ -247,8 +248,8 @@ extern "C" int pi_op_chunk_attention(const float * q, int64_t q_stride, const fl
     if (hpg * vdim > 256 * CA_MAXOUT || lds > 60 * 1024) { pi_set_error("pi_op_chunk_attention: %d query heads per key head of sizes %d / %d are beyond the kernel (LDS %zu bytes)", hpg, dim, vdim, lds); return -1; }
     const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
     const double visible = chunk > 0 ? std::min(acct, chunk) : acct;
-    PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention, dim3((unsigned) n_tok, (unsigned) kv_heads), dim3(256), lds,
-                 (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, chunk, heads, kv_heads, dim, vdim, n_kv, tile, out, out_stride,
+    PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention, dim3((unsigned) n_tok, (unsigned) kv_heads, (unsigned) ((heads / kv_heads + hpg - 1) / hpg)), dim3(256), lds,
+                 (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, chunk, heads, kv_heads, dim, vdim, n_kv, tile, hpg, out, out_stride,
                  dyn_dev, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
 }

@@ -36,6 +36,8 @@ llama_context::~llama_context() {
     if (pass_event) (void) hipEventDestroy(pass_event);
     for (uint8_t * b : pass_host) if (b) (void) hipHostFree(b);
     if (ctl_stream) { (void) hipStreamSynchronize(ctl_stream); (void) hipStreamDestroy(ctl_stream); }
+    if (branch_stream) { (void) hipStreamSynchronize(branch_stream); (void) hipStreamDestroy(branch_stream); }
+    for (hipEvent_t e : branch_events) if (e) (void) hipEventDestroy(e);
     if (abort_host) (void) hipHostFree(abort_host);
     if (hop_host) (void) hipHostFree(hop_host);
     pi_free(hop_dev);
@@ -131,6 +133,11 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
     pi_memset(ctx->lat_cache, 0, std::max<size_t>(lat * 4, 16), nullptr); pi_memset(ctx->rec_state, 0, std::max<size_t>(rec * 4, 16), nullptr);
     if (positions) { if (!(ctx->cell_pos = (int32_t *) dev((size_t) 4 * ctx->n_ctx)) || !(ctx->h_out2 = (float *) dev((size_t) 4 * nb * width)) || !(ctx->ssd_dt = (float *) dev((size_t) 4 * nb * step_w))) return false; pi_memset(ctx->cell_pos, 0, (size_t) 4 * ctx->n_ctx, nullptr); }
     if (hp.depth_average && !(ctx->hist = (float *) dev((size_t) 4 * (hp.hybrid.size() + 1) * nb * width))) return false;
+    if (positions && getenv("PI_BRANCH_STREAMS") && !strcmp(getenv("PI_BRANCH_STREAMS"), "1")) {            // (opt-in: measured at 4 % of a token's GPU time at width 2048; by default both branches follow each other on the context's stream)
+        if (hipStreamCreateWithFlags(&ctx->branch_stream, hipStreamNonBlocking) != hipSuccess) { err = "hipStreamCreate(branch) failed"; return false; }
+        ctx->branch_events.assign(2 * hp.hybrid.size(), nullptr);
+        for (hipEvent_t & e : ctx->branch_events) if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) { err = "hipEventCreate(branch) failed"; return false; }
+    }
     if (!(ctx->x = (float *) dev((size_t) 4 * nb * width)) || !(ctx->nx = (float *) dev((size_t) 4 * nb * width)) || !(ctx->h_out = (float *) dev((size_t) 4 * nb * width)) ||
         !(ctx->h_in = (float *) dev((size_t) 4 * nb * in_w)) || !(ctx->h_att = (float *) dev((size_t) 4 * nb * att_w)) || !(ctx->moe_up = (float *) dev((size_t) 4 * nb * up_w)) ||
         !(ctx->moe_w = (float *) dev((size_t) 4 * nb * sel_w)) || !(ctx->moe_dn = (float *) dev((size_t) 4 * nb * sel_w * width)) || !(ctx->moe_idx = (int32_t *) dev((size_t) 4 * idx_n)) || !(ctx->moe_sel = (int32_t *) dev((size_t) 4 * nb * sel_w)) || (ctx->slots && !(ctx->rec_dev = (int32_t *) dev((size_t) 4 * nb))) ||
@@ -309,6 +316,9 @@ static bool forward_parallel_mixer(llama_context * ctx, const pi_hybrid_layer & 
     float * kc = ctx->lat_cache + ctx->lat_off[il], * vc = kc + (size_t) ctx->n_ctx * gd;
     float * ssm = ctx->rec_state + ctx->rec_off[il], * conv_state = ssm + (size_t) ctx->slots->size() * R.heads * R.state * R.vdim;
     OP_OK(pi_op_dense(W.w_in, N, width, n_tok, P, pw, PI_ACT_NONE, pw, PI_ACT_NONE, ex, s));
+    // the recurrence branch goes to the branch stream (behind the projection), the attention branch stays; they meet again in front of the output projection
+    hipStream_t s_main = s, s2 = ctx->branch_stream ? ctx->branch_stream : s;
+    if (ctx->branch_stream && (hipEventRecord(ctx->branch_events[2 * il], s_main) != hipSuccess || hipStreamWaitEvent(s2, ctx->branch_events[2 * il], 0) != hipSuccess)) { ctx->last_error = "fork of the mixer's branches failed"; return false; }
     // attention branch (its output already carries the branch's factor)
     OP_OK(pi_op_qkv_prepare(P, P + hd, P + hd + gd, pw, W.q_norm, W.k_norm, eps, A.heads, A.kv_heads, A.dim, A.vdim, W.rotary, ctx->pos_dev, n_tok, Q, hd, kc, vc, ctx->cell_pos, ctx->dyn_dev, s));
     OP_OK(pi_op_chunk_attention(Q, hd, kc, vc, ctx->cell_pos, ctx->mask_dev, ctx->pos_dev, W.head_bias, P + hd + gd + gv, pw, PI_ACT_SIGMOID, A.scale, H.left_scale, A.chunk, A.heads, A.kv_heads, A.dim, A.vdim, n_tok, n_kv,
@@ -318,10 +328,11 @@ static bool forward_parallel_mixer(llama_context * ctx, const pi_hybrid_layer & 
     const float * R0 = P + A.in_rows();                                   // z | x B C | dt
     float * dt = ctx->ssd_dt, * decay = dt + (size_t) nb * R.heads;
     OP_OK(pi_op_causal_conv_steps(R0 + inner, pw, R.channels(), R.conv, W.conv_w, W.conv_b, conv_state, ctx->rec_dev, n_tok, PI_ACT_SILU, C, R.channels(),
-                                  R0 + inner + R.channels(), pw, W.dt_bias, W.a_log, R.heads, dt, decay, s));
+                                  R0 + inner + R.channels(), pw, W.dt_bias, W.a_log, R.heads, dt, decay, s2));
     OP_OK(pi_op_linear_attention_ex(C + inner + gn, C + inner, C, R.channels(), R.heads, R.groups, R.state, R.vdim, nullptr, decay, dt, R.heads, W.skip, ssm, ctx->rec_dev, n_tok, ctx->slots->size(),
-                                    ctx->rec_scratch, ctx->rec_scratch_floats, S, ow, s));
-    OP_OK(pi_op_gate_group_norm(S, ow, R0, pw, W.mix_norm, eps, H.right_scale, inner, R.norm_groups, n_tok, S, ow, s));
+                                    ctx->rec_scratch, ctx->rec_scratch_floats, S, ow, s2));
+    OP_OK(pi_op_gate_group_norm(S, ow, R0, pw, W.mix_norm, eps, H.right_scale, inner, R.norm_groups, n_tok, S, ow, s2));
+    if (ctx->branch_stream && (hipEventRecord(ctx->branch_events[2 * il + 1], s2) != hipSuccess || hipStreamWaitEvent(s_main, ctx->branch_events[2 * il + 1], 0) != hipSuccess)) { ctx->last_error = "join of the mixer's branches failed"; return false; }
     trace(ctx, "ssd", (int) il, S, inner, n_tok, ow);
     OP_OK(pi_op_dense(W.w_o, O, ow, n_tok, ctx->h_out, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));          // a * W_o att + b * W_o' rec
     return true;

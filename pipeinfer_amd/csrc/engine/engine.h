@@ -212,6 +212,9 @@ struct llama_context {
     // lightning layer (slots = state_slots), both at per-layer offsets into one allocation each
     float * lat_cache = nullptr, * rec_state = nullptr; std::vector<size_t> lat_off, rec_off;
     int32_t * cell_pos = nullptr;                             // position of every cell's token, on the device (mixers that look at positions besides the mask: chunks)
+    // a mixer's two branches do not depend on each other between the in- and the out-projection: with PI_BRANCH_STREAMS=1 the second one runs on a stream of its own (forked and joined
+    // by events, inside the captured graph as well as in eager launches) so that its small dependent kernels overlap the first one's
+    hipStream_t branch_stream = nullptr; std::vector<hipEvent_t> branch_events;     // [2 * layer]: fork, join
     float * hist = nullptr, * h_out2 = nullptr, * ssd_dt = nullptr;   // depth average: the stream after the embedding and after every layer [n_layer + 1][n_batch][width]; second branch output; step sizes | decays
     std::unique_ptr<pi::state_slots> slots; int n_state_slots = 8;
     int32_t * rec_dev = nullptr;                              // per token of the pass: state slot (| 1 << 30: start from zero)

@@ -531,6 +531,30 @@ def test_prompt_portions_and_decoding_agree_with_the_oracle(tmp_path, variant, e
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("exact", [True, False])
+def test_a_wider_model_with_long_passes(tmp_path, exact):
+    """sizes that reach the kernels' other paths: passes of 160 tokens (staged matrix-core products, grouped experts, the recurrence cut into pieces, the two-kernel convolution),
+    two tiles of visible keys per chunk, several value columns per thread; then portions and single tokens across the chunk borders at 48, 96, ... and 100, 200"""
+    layers = [O.parallel_layer(heads=6, kv_heads=3, dim=48, vdim=40, chunk=48, rot_dims=24, rot_base=500.0, scale=0.2, r_heads=6, r_vdim=32, state=40, groups=3, conv=4, norm_groups=2,
+                               mlp=O.routed_mlp(12, 3, 40, count=3, keep=2, shared=56)),
+              O.parallel_layer(heads=4, kv_heads=1, dim=72, vdim=80, chunk=100, rot_dims=72, rot_base=9000.0, scale=0.15, r_heads=8, r_vdim=24, state=72, groups=2, conv=3, norm_groups=4, mlp=O.dense_mlp(208)),
+              O.parallel_layer(heads=6, kv_heads=3, dim=48, vdim=40, chunk=48, rot_dims=24, rot_base=500.0, scale=0.2, r_heads=6, r_vdim=32, state=40, groups=3, conv=4, norm_groups=2,
+                               mlp=O.routed_mlp(12, 3, 40, count=3, keep=2, shared=56))]
+    m = small_model(seed=91, layers=layers, width=192, vocab=301)
+    rng = np.random.default_rng(17)
+    toks = [int(t) for t in rng.integers(0, 301, 260)]
+    want = O.run(m, toks)
+    e = Engine(tmp_path, m, n_ctx=288, n_batch=160, exact=exact)
+    whole = e.ctx.feed(toks, 0, 0)
+    assert within(logit_err(whole, want), exact)
+    e.ctx.seq_rm(0, -1, -1)
+    cut = np.concatenate([e.ctx.feed(toks[:91], 0, 0), e.ctx.feed(toks[91:97], 91, 0), e.ctx.feed(toks[97:198], 97, 0)] + [e.ctx.feed(toks[i:i + 1], i, 0) for i in range(198, 260)])
+    assert within(logit_err(cut, want), exact)
+    assert within(logit_err(cut, whole.astype(np.float64)), exact, 2e-5 if exact else 2e-2)
+    e.close()
+
+
+@pytest.mark.gpu
 def test_residual_stream_layer_by_layer(tmp_path):
     """models cut after 1, 2, ... layers give the oracle's logits, so the first wrong layer would be named (each cut model keeps its own depth-average factors)"""
     full = small_model(seed=4)

@@ -265,8 +265,8 @@ PI_API int pi_op_causal_conv_steps(const float * x_dev, int64_t x_stride, int ch
 PI_API int pi_op_ssd_steps(const float * raw_dev, int64_t raw_stride, const float * dt_bias_dev, const float * a_log_dev, int heads, int n_tok, float * dt_out_dev, float * decay_out_dev, void * stream);
 /* u = y * silu(z); out = u / rms(u over each of `groups` equal parts) * w * mult */
 PI_API int pi_op_gate_group_norm(const float * y_dev, int64_t y_stride, const float * z_dev, int64_t z_stride, const float * w_dev, float eps, float mult, int n, int groups, int n_tok, float * out_dev, int64_t out_stride, void * stream);
-/* router with sigmoid scores and a choice limited to groups: the outputs form n_groups equal groups of neighbours, a group's score is the sum of its two largest scores, only outputs of the
- * `keep` best groups can be chosen; the `top` largest scores among them win and are the weights (not renormalised) */
+/* router with sigmoid scores and a group-restricted choice: consecutive outputs are bundled into n_groups groups of equal size, a group is ranked by top1 + top2 of its members' scores, the
+ * choice is restricted to members of the `keep` highest-ranked groups; among them the `top` highest scores win, and those scores themselves are the mixing weights */
 PI_API int pi_op_moe_route_groups(const pi_weight * router, const float * x_dev, int64_t x_stride, int n_tok, int top, int n_groups, int keep, int exact, int32_t * sel_dev, float * selw_dev, void * stream);
 /* the grouped path with the expert's activation as a parameter (glu as for pi_op_moe_experts_act; up_dev is then [n_tok * top][2 * ff]) */
 PI_API int pi_op_moe_experts_grouped_act(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, int glu, const float * x_dev, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,

@@ -833,8 +833,8 @@ extern "C" int pi_op_latent_attention(const float * q, int64_t q_stride, const f
 
 // ---- routed feed-forward ------------------------------------------------------------------------------------------------------------------------------
 // one workgroup per token: logits of all router outputs (a wave per output), soft-max, choice = score + correction, `top` rounds of arg-max (lowest index wins a tie)
-// n_groups > 0: the scores are sigmoid(logit), the outputs form n_groups equal groups of neighbours, a group's score is the sum of its two largest scores and only outputs of the
-// `keep` best groups can be chosen (by their own score; lowest index wins a tie, among groups as among outputs)
+// n_groups > 0: the scores are sigmoid(logit), consecutive outputs are bundled into n_groups groups of equal size, a group is ranked by top1 + top2 of its members' scores, and the
+// choice is restricted to members of the `keep` highest-ranked groups (then by their own score; lowest index wins a tie, among groups as among outputs)
 __global__ void __launch_bounds__(256) k_moe_route(const uint16_t * __restrict__ router, int64_t width, int n_out, const float * __restrict__ corr, const float * __restrict__ x, int64_t xs,
                                                    int top, int exact, int vec, int n_groups, int keep, int32_t * __restrict__ sel, float * __restrict__ selw, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;

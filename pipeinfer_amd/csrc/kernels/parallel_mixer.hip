@@ -109,20 +109,22 @@ extern "C" int pi_op_qkv_prepare(const float * q, const float * k, const float *
 // head, value column), value rows read from the cache along the columns.
 // rows `cells[0 .. nl)` of a cache [cells][G][W] (head g) into LDS rows `pitch` floats apart.  Eight loads per thread are issued before the first LDS store: the compiler cannot
 // tell the cell list (LDS) from the tile (LDS) and would otherwise wait for every row's trip to memory before it reads the next cell number
+// RPW: rows a wave has in flight per round
+template <int RPW>
 static __device__ __forceinline__ void ca_stage(const float * __restrict__ cache, const int * cells, int nl, int G, int g, int W, int pitch, float * tile, int tid) {
     const int lane = tid & 63, wave = tid >> 6;
-    if (W <= 128) {                                                   // a wave per row, two columns per lane, four rows per round: no index arithmetic beyond adds
-        for (int r0 = wave; r0 < nl; r0 += 16) {
-            float tmp[8];
+    if (W <= 128) {                                                   // a wave per row, two columns per lane, RPW rows per round: no index arithmetic beyond adds
+        for (int r0 = wave; r0 < nl; r0 += 4 * RPW) {
+            float tmp[2 * RPW];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < RPW; u++) {
                 const int cc = r0 + u * 4;
                 const float * row = cache + ((int64_t) cells[min(cc, nl - 1)] * G + g) * W;
                 tmp[2 * u] = cc < nl && lane < W ? row[lane] : 0.0f;
                 tmp[2 * u + 1] = cc < nl && lane + 64 < W ? row[lane + 64] : 0.0f;
             }
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < RPW; u++) {
                 const int cc = r0 + u * 4;
                 if (cc < nl && lane < W) tile[cc * pitch + lane] = tmp[2 * u];
                 if (cc < nl && lane + 64 < W) tile[cc * pitch + lane + 64] = tmp[2 * u + 1];
@@ -148,6 +150,7 @@ static __device__ __forceinline__ void ca_stage(const float * __restrict__ cache
 #define CA_TILE 64                                // key rows staged at a time (fewer when a row is long: ca_tile)
 #define CA_SB 1                                   // blocks of 256 cells whose visibility is worked out in one round
 #define CA_MAXOUT 16                              // outputs (query head, value column) a thread accumulates: hpg * vdim <= 256 * CA_MAXOUT
+template <int RPW>
 __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * __restrict__ kc, const float * __restrict__ vc, const int32_t * __restrict__ cell_pos,
                                                          const uint32_t * __restrict__ mask, const int32_t * __restrict__ pos, const float * __restrict__ hbias, const float * __restrict__ gate, int64_t gs, int gate_act,
                                                          float scale, float out_mult, int chunk, int H, int G, int D, int V, int n_kv_arg, int tile, int hps, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
@@ -197,7 +200,7 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
         for (int l0 = 0; l0 < total; l0 += tile) {
             const int nl = min(tile, total - l0);
             if (l0) __syncthreads();                 // (the previous tile's values are no longer read)
-            ca_stage(kc, list + l0, nl, G, g, D, DP, ksh, tid);
+            ca_stage<RPW>(kc, list + l0, nl, G, g, D, DP, ksh, tid);
             __syncthreads();
             for (int i = tid; i < nl * hpg; i += 256) {
                 const int cc = i % nl, m = i / nl;
@@ -208,7 +211,7 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
             }
             __syncthreads();
             // the value rows take the key tile's place: all their loads are in flight together (read one by one in the sum below, every row would cost a trip to memory)
-            ca_stage(vc, list + l0, nl, G, g, V, V, ksh, tid);
+            ca_stage<RPW>(vc, list + l0, nl, G, g, V, V, ksh, tid);
             __syncthreads();
 #pragma unroll
             for (int oi = 0; oi < CA_MAXOUT; oi++) {
@@ -248,9 +251,11 @@ extern "C" int pi_op_chunk_attention(const float * q, int64_t q_stride, const fl
     if (hpg * vdim > 256 * CA_MAXOUT || lds > 60 * 1024) { pi_set_error("pi_op_chunk_attention: %d query heads per key head of sizes %d / %d are beyond the kernel (LDS %zu bytes)", hpg, dim, vdim, lds); return -1; }
     const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
     const double visible = chunk > 0 ? std::min(acct, chunk) : acct;
-    PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention, dim3((unsigned) n_tok, (unsigned) kv_heads, (unsigned) ((heads / kv_heads + hpg - 1) / hpg)), dim3(256), lds,
-                 (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, chunk, heads, kv_heads, dim, vdim, n_kv, tile, hpg, out, out_stride,
+#define CA_GO(R)     PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention<R>, dim3((unsigned) n_tok, (unsigned) kv_heads, (unsigned) ((heads / kv_heads + hpg - 1) / hpg)), dim3(256), lds, \
+                 (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, chunk, heads, kv_heads, dim, vdim, n_kv, tile, hpg, out, out_stride, \
                  dyn_dev, pi_abort_word());
+    CA_GO(4);                                                          // (deeper rounds were measured for single tokens: no gain, the registers they take cost as much as the trips they save)
+#undef CA_GO
     PI_CHECK_LAUNCH(); return 0;
 }
 

@@ -12,7 +12,7 @@ Mixer:       left_scale * attention(h) + right_scale * recurrence(h), both on th
               in the same block of `size` positions, else 0; nothing is normalised; head output * sigmoid(W_g h)_h; W_o.
   recurrence  W_in h = [z | x | B | C | dt]; (x, B, C) through a causal per-channel convolution of `conv` taps + bias, then silu; dt = softplus(dt + dt_bias);
               per head S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x (B, C of the head's group); (y * silu(z)) R-normed in `norm_groups` parts, * w; W_o.
-Feed-forward: dense  W_down relu(W_up h)^2;   routed  s = sigmoid(W_r h), group score = its two largest s, experts of the `keep` best groups compete, `top` largest s win
+Feed-forward: dense  W_down relu(W_up h)^2;   routed  s = sigmoid(W_r h), groups of consecutive experts ranked by top1 + top2 of s, members of the `keep` highest-ranked groups compete, the `top` highest s win
               with weight s (as it is); expert = W_down (silu(W_gate h) * W_up h); a shared expert of the same form is added for every token.
 Output:      cap * tanh((W_head LN_f(x)) / cap).
 """

@@ -87,6 +87,11 @@ def test_model_folder_is_read_and_described(tmp_path):
     mod.lib.llama_model_desc(mod.h, buf, 64)
     assert buf.value.lower().startswith(b"vikarax")
     mod.free()
+    for name, layers in VARIANTS.items():                          # descriptions without chunks, without a rotation, without groups, a shared expert or a feed-forward are read as well
+        if layers:
+            mv = small_model(seed=1, layers=layers, width=64 if name == "wide_heads" else 40)
+            write(str(tmp_path / name), mv)
+            LL.Model(str(tmp_path / name)).free()
 
 
 @pytest.mark.parametrize("breakage", ["type", "kv_heads", "rot", "groups", "keep", "kind", "norm_groups", "left_scale"])

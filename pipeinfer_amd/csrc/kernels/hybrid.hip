@@ -199,6 +199,85 @@ __global__ void __launch_bounds__(256) k_norm_chain_reg(const float * __restrict
 #pragma unroll
     for (int k = 0; k < NPT; k++) { const int i = threadIdx.x + k * 256; if (i < n) out_c[(int64_t) t * ocs + i] = (v[k] - mean_c) * inv_c * wv[k] + bv[k]; }
 }
+// ... and with 16-byte accesses: a thread owns NG groups of four neighbouring values (n % 4 == 0, rows 16-byte aligned, n <= 1024 * NG); one barrier per sum (each has its own LDS words)
+static __device__ __forceinline__ float hy_block_sum_once(float v, float * red) {
+    v = pi_lanes_sum<64>(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+template <int NG>
+__global__ void __launch_bounds__(256) k_norm_chain_vec(const float * __restrict__ a, int64_t as, float ca, const float * __restrict__ b, int64_t bs, float cb, const float * __restrict__ w,
+                                                        const float * __restrict__ bias, float eps, int n, const float * __restrict__ res, int64_t rs, float * __restrict__ out_a, int64_t oas,
+                                                        const float * __restrict__ hist, int64_t hist_stride, int n_hist, const float * __restrict__ coef, float * __restrict__ out_mix, int64_t oms,
+                                                        const float * __restrict__ w_c, const float * __restrict__ bias_c, float * __restrict__ out_c, int64_t ocs, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    __shared__ float red[4][4];
+    const int t = blockIdx.x;
+    const float * ar = a + (int64_t) t * as, * br = b ? b + (int64_t) t * bs : nullptr;
+    const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    float4 v[NG], wv[NG], bv[NG], rv[NG], mv[NG];
+    float sum = 0.0f;
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        const int i = (threadIdx.x + g * 256) * 4;
+        const bool ok = i < n;
+        float4 x = ok ? *(const float4 *) (ar + i) : zero;
+        x.x *= ca; x.y *= ca; x.z *= ca; x.w *= ca;
+        if (ok && br) { const float4 y = *(const float4 *) (br + i); x.x = fmaf(cb, y.x, x.x); x.y = fmaf(cb, y.y, x.y); x.z = fmaf(cb, y.z, x.z); x.w = fmaf(cb, y.w, x.w); }
+        v[g] = x; sum += (x.x + x.y) + (x.z + x.w);
+        wv[g] = ok ? *(const float4 *) (w + i) : zero;
+        bv[g] = ok && bias ? *(const float4 *) (bias + i) : zero;
+        rv[g] = ok && res ? *(const float4 *) (res + (int64_t) t * rs + i) : zero;
+        float4 m = zero;
+        if (ok) for (int j = 0; j < n_hist - 1; j++) {
+            const float c = coef[j]; const float4 h = *(const float4 *) (hist + (int64_t) j * hist_stride + (int64_t) t * n + i);
+            m.x = fmaf(c, h.x, m.x); m.y = fmaf(c, h.y, m.y); m.z = fmaf(c, h.z, m.z); m.w = fmaf(c, h.w, m.w);
+        }
+        mv[g] = m;
+    }
+    const float mean = hy_block_sum_once(sum, red[0]) / (float) n;
+    float ss = 0.0f;
+#pragma unroll
+    for (int g = 0; g < NG; g++) if ((threadIdx.x + g * 256) * 4 < n) {
+        const float d0 = v[g].x - mean, d1 = v[g].y - mean, d2 = v[g].z - mean, d3 = v[g].w - mean;
+        ss = fmaf(d0, d0, ss); ss = fmaf(d1, d1, ss); ss = fmaf(d2, d2, ss); ss = fmaf(d3, d3, ss);
+    }
+    const float inv = 1.0f / sqrtf(hy_block_sum_once(ss, red[1]) / (float) n + eps);
+    const float c_last = n_hist > 0 ? coef[n_hist - 1] : 0.0f;
+    float sum_c = 0.0f;
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        const int i = (threadIdx.x + g * 256) * 4;
+        if (i < n) {
+            float4 y = make_float4((v[g].x - mean) * inv * wv[g].x + bv[g].x, (v[g].y - mean) * inv * wv[g].y + bv[g].y, (v[g].z - mean) * inv * wv[g].z + bv[g].z, (v[g].w - mean) * inv * wv[g].w + bv[g].w);
+            if (res) { y.x = rv[g].x + y.x; y.y = rv[g].y + y.y; y.z = rv[g].z + y.z; y.w = rv[g].w + y.w; }
+            *(float4 *) (out_a + (int64_t) t * oas + i) = y;
+            if (n_hist > 0) {
+                y.x = fmaf(c_last, y.x, mv[g].x); y.y = fmaf(c_last, y.y, mv[g].y); y.z = fmaf(c_last, y.z, mv[g].z); y.w = fmaf(c_last, y.w, mv[g].w);
+                *(float4 *) (out_mix + (int64_t) t * oms + i) = y;
+            }
+            v[g] = y; sum_c += (y.x + y.y) + (y.z + y.w);
+        }
+    }
+    if (!w_c) return;
+#pragma unroll
+    for (int g = 0; g < NG; g++) { const int i = (threadIdx.x + g * 256) * 4; wv[g] = i < n ? *(const float4 *) (w_c + i) : zero; bv[g] = i < n && bias_c ? *(const float4 *) (bias_c + i) : zero; }
+    const float mean_c = hy_block_sum_once(sum_c, red[2]) / (float) n;
+    float ss_c = 0.0f;
+#pragma unroll
+    for (int g = 0; g < NG; g++) if ((threadIdx.x + g * 256) * 4 < n) {
+        const float d0 = v[g].x - mean_c, d1 = v[g].y - mean_c, d2 = v[g].z - mean_c, d3 = v[g].w - mean_c;
+        ss_c = fmaf(d0, d0, ss_c); ss_c = fmaf(d1, d1, ss_c); ss_c = fmaf(d2, d2, ss_c); ss_c = fmaf(d3, d3, ss_c);
+    }
+    const float inv_c = 1.0f / sqrtf(hy_block_sum_once(ss_c, red[3]) / (float) n + eps);
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        const int i = (threadIdx.x + g * 256) * 4;
+        if (i < n) *(float4 *) (out_c + (int64_t) t * ocs + i) = make_float4((v[g].x - mean_c) * inv_c * wv[g].x + bv[g].x, (v[g].y - mean_c) * inv_c * wv[g].y + bv[g].y,
+                                                                              (v[g].z - mean_c) * inv_c * wv[g].z + bv[g].z, (v[g].w - mean_c) * inv_c * wv[g].w + bv[g].w);
+    }
+}
 extern "C" int pi_op_layer_norm_mix(const float * a, int64_t a_stride, float ca, const float * b, int64_t b_stride, float cb, const float * w_dev, const float * bias_dev, float eps, int n, int n_tok,
                                     const float * residual, int64_t residual_stride, float * out, int64_t out_stride, void * stream) {
     return pi_op_norm_chain(a, a_stride, ca, b, b_stride, cb, w_dev, bias_dev, eps, n, n_tok, residual, residual_stride, out, out_stride, nullptr, 0, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, 0, stream);
@@ -214,7 +293,11 @@ extern "C" int pi_op_norm_chain(const float * a, int64_t a_stride, float ca, con
     const double bytes = 4.0 * n * n_tok * (3.0 + (b ? 1 : 0) + (residual ? 1 : 0) + n_hist + (w_next ? 2 : 0));
 #define NC_GO(K) PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, bytes, K, dim3((unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, a, a_stride, ca, b, b_stride, cb, w_dev, bias_dev, eps, n, residual, residual_stride, \
                               out_a, out_a_stride, hist, hist_stride, n_hist, coef_dev, out_mix, out_mix_stride, w_next, bias_next, out_next, out_next_stride, pi_abort_word())
-    if (n <= 1024) NC_GO(k_norm_chain_reg<4>); else if (n <= 2048) NC_GO(k_norm_chain_reg<8>); else if (n <= 4096) NC_GO(k_norm_chain_reg<16>); else if (n <= 8192) NC_GO(k_norm_chain_reg<32>); else NC_GO(k_norm_chain);
+    auto al = [](const void * p, int64_t stride) { return !p || (((uintptr_t) p % 16) == 0 && stride % 4 == 0); };
+    const bool vec = n % 4 == 0 && n <= 8192 && al(a, a_stride) && al(b, b_stride) && al(w_dev, 0) && al(bias_dev, 0) && al(residual, residual_stride) && al(out_a, out_a_stride) && al(hist, hist_stride) &&
+                     al(out_mix, out_mix_stride) && al(w_next, 0) && al(bias_next, 0) && al(out_next, out_next_stride);
+    if (vec) { if (n <= 1024) NC_GO(k_norm_chain_vec<1>); else if (n <= 2048) NC_GO(k_norm_chain_vec<2>); else if (n <= 4096) NC_GO(k_norm_chain_vec<4>); else NC_GO(k_norm_chain_vec<8>); }
+    else if (n <= 1024) NC_GO(k_norm_chain_reg<4>); else if (n <= 2048) NC_GO(k_norm_chain_reg<8>); else if (n <= 4096) NC_GO(k_norm_chain_reg<16>); else if (n <= 8192) NC_GO(k_norm_chain_reg<32>); else NC_GO(k_norm_chain);
 #undef NC_GO
     PI_CHECK_LAUNCH(); return 0;
 }
